@@ -28,7 +28,11 @@ setup(
             sources=SOURCES,
             extra_compile_args={
                 "cxx": ["-O3", "-std=c++17"],
-                "nvcc": ["-O3", "-std=c++17", "--offload-arch=gfx950"],
+                # packed-fp32 instruction selection is switched off for
+                # every kernel of the extension
+                "nvcc": ["-O3", "-std=c++17", "--offload-arch=gfx950",
+                         "-Xclang", "-target-feature",
+                         "-Xclang", "-packed-fp32-ops"],
             },
         )
     ],

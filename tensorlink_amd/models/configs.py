@@ -109,6 +109,10 @@ class ModelConfig:
         if not isinstance(cfg, dict):
             cfg = {k: getattr(cfg, k) for k in dir(cfg) if not k.startswith("_")
                    if not callable(getattr(cfg, k, None))}
+        if cfg.get("architecture") in ("Kepusun", "kepusun"):
+            # layered family: the config lists its layers one by one
+            from tensorlink_amd.models.kepusun import KepusunConfig
+            return KepusunConfig.from_dict(cfg, name=name)
         if "architecture" in cfg and "architectures" not in cfg:
             # our own to_json round-trip (save_hf_checkpoint writes it)
             known = {f.name for f in dataclasses.fields(cls)}

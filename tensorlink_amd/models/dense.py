@@ -451,4 +451,7 @@ def _stage_class(config: ModelConfig):
     if config.architecture == "neox":
         from tensorlink_amd.models.neox import NeoxStageModel
         return NeoxStageModel
+    if config.architecture == "kepusun":
+        from tensorlink_amd.models.kepusun import KepusunStageModel
+        return KepusunStageModel
     return StageModel

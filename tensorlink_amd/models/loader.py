@@ -122,6 +122,11 @@ def load_stage_from_checkpoint(stage: StageModel, ckpt_dir: str,
         n = load_neox_hf_weights(stage, ckpt_dir, dtype=dtype)
         stage.to(device=device, dtype=dtype)
         return n
+    if arch == "kepusun":
+        from tensorlink_amd.models.kepusun import load_kepusun_weights
+        n = load_kepusun_weights(stage, ckpt_dir, dtype=dtype)
+        stage.to(device=device, dtype=dtype)
+        return n
     from safetensors import safe_open
 
     index_path = os.path.join(ckpt_dir, "model.safetensors.index.json")
@@ -161,6 +166,10 @@ def load_stage_from_checkpoint(stage: StageModel, ckpt_dir: str,
 def init_random_stage(stage: StageModel, device="cpu", dtype=torch.bfloat16,
                       seed: int = 0) -> StageModel:
     """Deterministic scaled-normal init directly on the target device."""
+    if stage.config.architecture == "kepusun":
+        from tensorlink_amd.models.kepusun import init_kepusun_random
+        init_kepusun_random(stage, seed=seed)
+        return stage.to(device=device, dtype=dtype)
     gen_dev = device if str(device).startswith("cuda") else "cpu"
     g = torch.Generator(device=gen_dev)
     g.manual_seed(seed)

@@ -1,0 +1,235 @@
+"""Building blocks beyond the Llama shape: Dynamic-Tanh norm,
+hyper-connected residual streams, matrix-memory (mLSTM) mixer,
+differential attention with cross-layer KV sharing, and a group-limited
+top-k mixture of experts with squared-ReLU experts.
+
+Every block takes its sizes and constants as constructor arguments, runs
+on flat ragged batches (:class:`tensorlink_amd.ops.mixers.RaggedMeta`) and
+keeps its per-sequence memory in the slot/page cache handed to it
+(:class:`tensorlink_amd.models.paged.HybridSlotCache`), so a model file
+only assembles them by configuration.
+
+Precision: what feeds a norm, a router, a gate of a recurrence, a score or
+the residual is fp32 whatever the serving dtype; the big projections and
+expert GEMMs run in the serving dtype with fp32 accumulation.
+"""
+
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from tensorlink_amd import ops
+from tensorlink_amd.models.dense import TLLinear
+from tensorlink_amd.ops import mixers as mx
+
+
+class _F32Cache:
+    """fp32 contiguous copies of small parameters, rebuilt when the
+    parameter is written or moved (the module may be stored in bf16)."""
+
+    def _f32(self, name: str) -> torch.Tensor:
+        p = getattr(self, name)
+        store = self.__dict__.setdefault("_f32_store", {})
+        key = (p.data_ptr(), p._version, p.device, p.dtype)
+        hit = store.get(name)
+        if hit is None or hit[0] != key:
+            hit = (key, p.detach().float().contiguous())
+            store[name] = hit
+        return hit[1]
+
+
+class DynamicTanh(nn.Module, _F32Cache):
+    """y = tanh(alpha * x) * weight + bias; no mean, no variance."""
+
+    def __init__(self, width: int):
+        super().__init__()
+        self.weight = nn.Parameter(torch.ones(width))
+        self.bias = nn.Parameter(torch.zeros(width))
+        self.alpha = nn.Parameter(torch.ones(()))
+
+    def params(self):
+        return (self._f32("alpha").reshape(1), self._f32("weight"),
+                self._f32("bias"))
+
+
+class HyperConnection(nn.Module, _F32Cache):
+    """Read weights ``inw`` [ns], write weights ``out`` [ns] and stream
+    mixing matrix ``mix`` [from, to] of one sublayer."""
+
+    def __init__(self, streams: int):
+        super().__init__()
+        self.inw = nn.Parameter(torch.full((streams,), 1.0 / streams))
+        self.out = nn.Parameter(torch.ones(streams))
+        self.mix = nn.Parameter(torch.eye(streams))
+
+
+class MLSTMMixer(nn.Module, _F32Cache):
+    """Matrix-memory mixer: fused q|k|v|g projection, fp32 soft-capped
+    gates, the slot-state recurrence kernel, output projection."""
+
+    kind = "mlstm"
+
+    def __init__(self, width: int, heads: int, dim: int, vdim: int,
+                 gate_cap: float, eps: float):
+        super().__init__()
+        self.H, self.D, self.V = heads, dim, vdim
+        self.cap, self.eps = float(gate_cap), float(eps)
+        hd, hv = heads * dim, heads * vdim
+        self.offs = (0, hd, 2 * hd, 2 * hd + hv)
+        self.proj = TLLinear(width, 2 * hd + 2 * hv, bias=False)
+        self.gate = nn.Linear(width, 2 * heads, bias=True)   # input | forget
+        self.norm = nn.Parameter(torch.ones(hv))
+        self.o_proj = TLLinear(hv, width, bias=False)
+
+    def cache_spec(self):
+        return {"kind": "mlstm", "H": self.H, "D": self.D, "V": self.V}
+
+    def forward(self, h, meta, cache, layer_idx):
+        proj = self.proj(h)
+        gw = self.gate.weight
+        if gw.dtype != torch.float32:
+            store = self.__dict__.setdefault("_gate32", None)
+            key = (gw.data_ptr(), gw._version, self.gate.bias._version)
+            if store is None or store[0] != key:
+                store = (key, gw.detach().float(),
+                         self.gate.bias.detach().float())
+                self.__dict__["_gate32"] = store
+            gates = F.linear(h.float(), store[1], store[2])
+        else:
+            gates = F.linear(h.float(), gw, self.gate.bias)
+        S, n, m = cache.state[layer_idx]
+        o = mx.mlstm_scan(proj, self.offs, gates, self._f32("norm"), S, n, m,
+                          meta, self.H, self.D, self.V, self.cap, self.eps)
+        return self.o_proj(o)
+
+
+class DiffAttention(nn.Module, _F32Cache):
+    """Two-map (differential) softmax attention over the paged pool, GQA,
+    position-free scores. ``kv_from`` = index of an earlier layer whose
+    key/value pools this layer reads instead of projecting its own."""
+
+    kind = "attention"
+
+    def __init__(self, width: int, heads: int, kv_heads: int, dim: int,
+                 vdim: int, scale: float, diff: float, eps: float,
+                 kv_from: Optional[int] = None):
+        super().__init__()
+        assert heads % kv_heads == 0
+        self.H, self.G, self.D, self.V = heads, kv_heads, dim, vdim
+        self.scale, self.diff, self.eps = float(scale), float(diff), float(eps)
+        self.kv_from = kv_from
+        self.q_cols = heads * 2 * dim
+        self.k_cols = 0 if kv_from is not None else kv_heads * 2 * dim
+        self.v_cols = 0 if kv_from is not None else kv_heads * vdim
+        self.qkv = TLLinear(width, self.q_cols + self.k_cols + self.v_cols,
+                            bias=False)
+        self.lq1 = nn.Parameter(torch.zeros(dim))
+        self.lk1 = nn.Parameter(torch.zeros(dim))
+        self.lq2 = nn.Parameter(torch.zeros(dim))
+        self.lk2 = nn.Parameter(torch.zeros(dim))
+        self.o_proj = TLLinear(heads * vdim, width, bias=False)
+
+    def cache_spec(self):
+        if self.kv_from is not None:
+            return {"kind": "kv_ref", "src": self.kv_from}
+        return {"kind": "kv", "G": self.G, "DK": 2 * self.D, "V": self.V}
+
+    def lam(self) -> torch.Tensor:
+        """exp(lq1.lk1) - exp(lq2.lk2) + diff as a 1-element fp32 tensor,
+        recomputed only when a lambda parameter changes."""
+        key = tuple((p.data_ptr(), p._version) for p in
+                    (self.lq1, self.lk1, self.lq2, self.lk2))
+        hit = self.__dict__.get("_lam")
+        if hit is None or hit[0] != key:
+            v = (torch.exp((self.lq1.float() * self.lk1.float()).sum())
+                 - torch.exp((self.lq2.float() * self.lk2.float()).sum())
+                 + self.diff).reshape(1).detach()
+            hit = (key, v)
+            self.__dict__["_lam"] = hit
+        return hit[1]
+
+    def forward(self, h, meta, cache, layer_idx):
+        proj = self.qkv(h)
+        src = layer_idx if self.kv_from is None else self.kv_from
+        kpool, vpool = cache.k[src], cache.v[src]
+        if self.kv_from is None:
+            mx.kv_append(proj, self.q_cols, self.q_cols + self.k_cols,
+                         kpool, vpool, meta)
+        o = mx.diff_attention(proj, 0, kpool, vpool, meta, self.lam(),
+                              self.H, self.D, self.scale, self.diff,
+                              self.eps)
+        return self.o_proj(o)
+
+
+class GroupLimitedMoE(nn.Module, _F32Cache):
+    """Mixture of two-matrix experts (down(relu(up x)^2), no biases) under
+    a softmax router with group-limited top-k selection."""
+
+    def __init__(self, width: int, ff: int, experts: int, top: int,
+                 n_groups: int, keep_groups: int, route_scale: float):
+        super().__init__()
+        assert experts % n_groups == 0 and keep_groups <= n_groups
+        assert top <= keep_groups * (experts // n_groups)
+        self.W, self.ff, self.E, self.top = width, ff, experts, top
+        self.n_groups, self.keep = n_groups, keep_groups
+        self.route_scale = float(route_scale)
+        self.router = nn.Parameter(torch.zeros(experts, width))
+        self.up = nn.Parameter(torch.zeros(experts, ff, width))
+        self.down = nn.Parameter(torch.zeros(experts, width, ff))
+
+    def _grouped_ok(self, h) -> bool:
+        return (h.is_cuda and h.dtype == torch.bfloat16
+                and ops.extension_loaded()
+                and self.W % 64 == 0 and self.ff % 64 == 0)
+
+    def _tables(self, dev):
+        key = (self.up.data_ptr(), self.down.data_ptr(), str(dev))
+        hit = self.__dict__.get("_ptrs")
+        if hit is None or hit[0] != key:
+            mk = lambda p: torch.tensor(
+                [p[e].data_ptr() for e in range(self.E)],
+                dtype=torch.int64, device=dev)
+            hit = (key, mk(self.up), mk(self.down))
+            self.__dict__["_ptrs"] = hit
+        return hit[1], hit[2]
+
+    def forward(self, h):
+        T = h.shape[0]
+        logits = F.linear(h.float(), self._f32("router"))
+        w, idx = mx.group_limited_router(logits, self.top, self.n_groups,
+                                         self.keep, self.route_scale)
+        if self._grouped_ok(h):
+            # grouped expert GEMMs over expert-sorted (token, choice) pairs
+            # (ops/csrc/moe_gemm.hip); fixed-order fp32 combine, no atomics
+            C = ops._require_ext()
+            dev = h.device
+            up_p, down_p = self._tables(dev)
+            fi = idx.reshape(-1)
+            order = fi.argsort(stable=True)
+            counts = torch.zeros(self.E, device=dev, dtype=torch.long)
+            counts.scatter_add_(0, fi, torch.ones_like(fi))
+            seg = torch.zeros(self.E + 1, device=dev, dtype=torch.int32)
+            seg[1:] = counts.cumsum(0)
+            pair_tok = (order // self.top).to(torch.int32)
+            a = C.moe_gemm(h.contiguous(), pair_tok, seg, up_p, None,
+                           self.ff, False)
+            a = mx.relu_squared(a)
+            y = C.moe_gemm(a, None, seg, down_p, None, self.W, False)
+            y = y.float() * w.reshape(-1)[order].unsqueeze(1)
+            inv = torch.empty_like(order)
+            inv[order] = torch.arange(order.numel(), device=dev,
+                                      dtype=order.dtype)
+            return y[inv].view(T, self.top, self.W).sum(1).to(h.dtype)
+        out = torch.zeros(T, self.W, device=h.device, dtype=torch.float32)
+        for e in range(self.E):
+            tok, choice = (idx == e).nonzero(as_tuple=True)
+            if tok.numel() == 0:
+                continue
+            a = mx.relu_squared(F.linear(h[tok], self.up[e]))
+            out.index_add_(0, tok, F.linear(a, self.down[e]).float()
+                           * w[tok, choice, None])
+        return out.to(h.dtype)

@@ -148,7 +148,73 @@ class DynamicPagedKVCache(PagedKVCache):
             self.release_slot(s)
 
 
+class HybridSlotCache(DynamicPagedKVCache):
+    """Slot cache for models whose layers differ: per layer either paged
+    key/value pools of that layer's own head sizes, a reference to an
+    earlier layer's pools (cross-layer KV sharing), or fp32 recurrent
+    state indexed by slot.
+
+    ``specs[l]`` is ``{"kind": "kv", "G", "DK", "V"}``,
+    ``{"kind": "kv_ref", "src": j}`` or ``{"kind": "mlstm", "H", "D",
+    "V"}``. ``k[l]`` / ``v[l]`` are [pool_pages, G, PAGE, DK|V] (None for
+    recurrent layers, the source's tensors for references); ``state[l]``
+    is (S [slots, H, D, V], n [slots, H, D], m [slots, H]) or None. Pages
+    are leased and returned exactly as in :class:`DynamicPagedKVCache`;
+    recurrent state needs no clearing on release because the kernels start
+    a sequence with no cached tokens from zeros."""
+
+    SWAPPABLE = False           # host-swap preemption not implemented
+
+    def __init__(self, specs, slots: int, pool_pages: int, max_seq: int,
+                 device, dtype=torch.bfloat16):
+        self.specs = list(specs)
+        self.k, self.v, self.state = [], [], []
+        for sp in self.specs:
+            if sp["kind"] == "kv":
+                self.k.append(torch.zeros(pool_pages, sp["G"], PAGE,
+                                          sp["DK"], device=device,
+                                          dtype=dtype))
+                self.v.append(torch.zeros(pool_pages, sp["G"], PAGE,
+                                          sp["V"], device=device,
+                                          dtype=dtype))
+                self.state.append(None)
+            elif sp["kind"] == "kv_ref":
+                self.k.append(self.k[sp["src"]])
+                self.v.append(self.v[sp["src"]])
+                self.state.append(None)
+            else:
+                f32 = dict(device=device, dtype=torch.float32)
+                self.k.append(None)
+                self.v.append(None)
+                self.state.append((
+                    torch.zeros(slots, sp["H"], sp["D"], sp["V"], **f32),
+                    torch.zeros(slots, sp["H"], sp["D"], **f32),
+                    torch.zeros(slots, sp["H"], **f32)))
+        self.seq_lens = torch.zeros(slots, device=device, dtype=torch.int32)
+        self.pages_per_seq = max(1, (max_seq + PAGE - 1) // PAGE)
+        self.max_seq = self.pages_per_seq * PAGE
+        self.batch = slots
+        self.allocator = PageAllocator(pool_pages)
+        self.table = torch.zeros(slots, self.pages_per_seq, device=device,
+                                 dtype=torch.int32)
+        self._slot_pages = [[] for _ in range(slots)]
+        self.slot_ids = list(range(slots))
+
+    def slice(self, s: int, e: int):
+        """View over slots s..e-1 (micro-batch split of a rectangular
+        batch); pools and state are shared by reference."""
+        view = object.__new__(HybridSlotCache)
+        view.__dict__.update(self.__dict__)
+        view.table = self.table[s:e]
+        view.seq_lens = self.seq_lens[s:e]
+        view.slot_ids = self.slot_ids[s:e]
+        view.batch = e - s
+        return view
+
+
 def kv_slice_paged(cache: PagedKVCache, s: int, e: int) -> PagedKVCache:
+    if isinstance(cache, HybridSlotCache):
+        return cache.slice(s, e)
     view = object.__new__(PagedKVCache)
     view.k = cache.k                       # pools shared
     view.v = cache.v

@@ -1,0 +1,174 @@
+// Matrix-memory (mLSTM) recurrence over ragged sequences (gfx950).
+//
+// Per head the state is a matrix S [D, V], a normaliser n [D] and a running
+// log-scale m, all fp32 and resident in a slot pool between steps. For a
+// token with log gates (li, lf), key k, value v and scaled query q:
+//     m' = max(lf + m, li)
+//     S' = exp(lf + m - m') S + exp(li - m') k v^T       (n' likewise, v = 1)
+//     o  = S'^T q / (max(|n' . q|, exp(-m')) + 1e-6)
+// followed, fused here, by the per-head unit-RMS norm, the norm weight and
+// the sigmoid output gate. The raw gate pre-activations arrive in fp32 and
+// are soft-capped in-kernel: li = cap*tanh(gi/cap),
+// lf = logsigmoid(cap*tanh(gf/cap)).
+//
+// One block serves one (sequence, head) and walks the sequence's tokens in
+// order, so the same kernel is the decode step (one token) and the exact
+// sequential prefill. Thread c < V owns column c of S in registers; thread
+// c == V owns n (the column a constant value 1 would produce), so n . q
+// falls out of the same dot product. A sequence whose cached length is zero
+// starts from the zero state without reading its slot: a reused slot needs
+// no clearing.
+
+#include "common.hpp"
+
+namespace {
+
+template <typename T> DEVINLINE float ldv(const T* p);
+template <> DEVINLINE float ldv<float>(const float* p) { return *p; }
+template <> DEVINLINE float ldv<bf16>(const bf16* p) { return bf2f(*p); }
+template <typename T> DEVINLINE void stv(T* p, float v);
+template <> DEVINLINE void stv<float>(float* p, float v) { *p = v; }
+template <> DEVINLINE void stv<bf16>(bf16* p, float v) { *p = f2bf(v); }
+
+DEVINLINE float log_sigmoid(float x) {
+  return fminf(x, 0.f) - log1pf(expf(-fabsf(x)));
+}
+
+template <typename T, int DMAX>
+__global__ void mlstm_seq_kernel(
+    const T* __restrict__ proj, int ld, int q_off, int k_off, int v_off,
+    int g_off,
+    const float* __restrict__ gates,   // [Ttot, 2H] raw (input | forget)
+    const float* __restrict__ norm_w,  // [H*V]
+    float* __restrict__ S_pool,        // [slots, H, D, V]
+    float* __restrict__ n_pool,        // [slots, H, D]
+    float* __restrict__ m_pool,        // [slots, H]
+    const int* __restrict__ cu, const int* __restrict__ slots,
+    const int* __restrict__ pos0, T* __restrict__ out, int H, int D, int V,
+    float cap, float qscale, float eps) {
+  extern __shared__ float lds[];
+  const int h = blockIdx.x, b = blockIdx.y;
+  const int c = threadIdx.x;
+  const int nw = blockDim.x / WAVE_SIZE;
+  const int lane = c & (WAVE_SIZE - 1), wave = c / WAVE_SIZE;
+  // lds: q[2][D] | k[2][D] | red[2][nw + 1]
+  float* lq = lds;
+  float* lk = lds + 2 * D;
+  float* red = lds + 4 * D;
+
+  const int t0 = cu[b], t1 = cu[b + 1];
+  if (t0 >= t1) return;
+  const int slot = slots[b];
+  const bool fresh = pos0[b] == 0;
+  const bool is_col = c < V, is_n = c == V;
+
+  float s[DMAX];
+  float* S_base = S_pool + ((int64_t)slot * H + h) * (int64_t)D * V;
+  float* n_base = n_pool + ((int64_t)slot * H + h) * D;
+#pragma unroll
+  for (int d = 0; d < DMAX; ++d) {
+    float v = 0.f;
+    if (!fresh && d < D) {
+      if (is_col) v = S_base[(int64_t)d * V + c];
+      else if (is_n) v = n_base[d];
+    }
+    s[d] = v;
+  }
+  float m = fresh ? 0.f : m_pool[(int64_t)slot * H + h];
+
+  for (int t = t0; t < t1; ++t) {
+    const int par = (t - t0) & 1;
+    const T* row = proj + (int64_t)t * ld;
+    for (int d = c; d < D; d += blockDim.x) {
+      lq[par * D + d] = ldv<T>(row + q_off + h * D + d) * qscale;
+      lk[par * D + d] = ldv<T>(row + k_off + h * D + d);
+    }
+    const float gi = gates[(int64_t)t * 2 * H + h];
+    const float gf = gates[(int64_t)t * 2 * H + H + h];
+    const float li = cap * tanhf(gi / cap);
+    const float lf = log_sigmoid(cap * tanhf(gf / cap));
+    const float m_new = fmaxf(lf + m, li);
+    const float a = expf(lf + m - m_new);
+    const float bb = expf(li - m_new);
+    m = m_new;
+    const float vc = is_col ? ldv<T>(row + v_off + h * V + c)
+                            : (is_n ? 1.f : 0.f);
+    __syncthreads();
+    float num = 0.f;
+    const float bv = bb * vc;
+    const float* qq = lq + par * D;
+    const float* kk = lk + par * D;
+#pragma unroll
+    for (int d = 0; d < DMAX; ++d) {
+      if (d < D) {
+        s[d] = a * s[d] + bv * kk[d];
+        num += s[d] * qq[d];
+      }
+    }
+    const float sq = wave_reduce_sum(is_col ? num * num : 0.f);
+    float* rr = red + par * (nw + 1);
+    if (lane == 0) rr[wave] = sq;
+    if (is_n) rr[nw] = num;
+    __syncthreads();
+    float ss = 0.f;
+    for (int w = 0; w < nw; ++w) ss += rr[w];
+    const float den = fmaxf(fabsf(rr[nw]), expf(-m)) + 1e-6f;
+    if (is_col) {
+      const float o = num / den;
+      const float r = rsqrtf(ss / (den * den) / (float)V + eps);
+      const float g = ldv<T>(row + g_off + h * V + c);
+      const float sg = 1.f / (1.f + expf(-g));
+      stv<T>(out + (int64_t)t * H * V + h * V + c,
+             o * r * norm_w[h * V + c] * sg);
+    }
+  }
+#pragma unroll
+  for (int d = 0; d < DMAX; ++d) {
+    if (d < D) {
+      if (is_col) S_base[(int64_t)d * V + c] = s[d];
+      else if (is_n) n_base[d] = s[d];
+    }
+  }
+  if (c == 0) m_pool[(int64_t)slot * H + h] = m;
+}
+
+}  // namespace
+
+extern "C" {
+
+// returns 0 on success, 1 if the shape is outside what the kernel serves
+int tl_mlstm_seq(const void* proj, int ld, int q_off, int k_off, int v_off,
+                 int g_off, const void* gates, const void* norm_w, void* S,
+                 void* n, void* m, const void* cu, const void* slots,
+                 const void* pos0, void* out, int B, int H, int D, int V,
+                 float cap, float qscale, float eps, int is_f32,
+                 hipStream_t stream) {
+  if (D > 256 || V + 1 > 1024 || B < 1) return 1;
+  const int nt = ((V + 1 + WAVE_SIZE - 1) / WAVE_SIZE) * WAVE_SIZE;
+  const int nw = nt / WAVE_SIZE;
+  const size_t smem = sizeof(float) * (4 * D + 2 * (nw + 1));
+  dim3 grid(H, B), block(nt);
+#define TL_ML_LAUNCH(TT, DM)                                                 \
+  hipLaunchKernelGGL((mlstm_seq_kernel<TT, DM>), grid, block, smem, stream,  \
+                     (const TT*)proj, ld, q_off, k_off, v_off, g_off,        \
+                     (const float*)gates, (const float*)norm_w, (float*)S,   \
+                     (float*)n, (float*)m, (const int*)cu,                   \
+                     (const int*)slots, (const int*)pos0, (TT*)out, H, D, V, \
+                     cap, qscale, eps)
+#define TL_ML_D(TT)                                  \
+  if (D <= 16) TL_ML_LAUNCH(TT, 16);                 \
+  else if (D <= 32) TL_ML_LAUNCH(TT, 32);            \
+  else if (D <= 64) TL_ML_LAUNCH(TT, 64);            \
+  else if (D <= 128) TL_ML_LAUNCH(TT, 128);          \
+  else TL_ML_LAUNCH(TT, 256);
+  if (is_f32) {
+    TL_ML_D(float)
+  } else {
+    TL_ML_D(bf16)
+  }
+#undef TL_ML_D
+#undef TL_ML_LAUNCH
+  return 0;
+}
+
+}  // extern "C"

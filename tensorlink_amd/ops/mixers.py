@@ -1,0 +1,259 @@
+"""Sequence-mixer ops over ragged batches: hyper-connection + Dynamic-Tanh,
+matrix-memory (mLSTM) recurrence with slot-resident state, differential
+attention over the paged KV pool, group-limited top-k routing.
+
+Same dispatch policy as the rest of :mod:`tensorlink_amd.ops`: tensors on
+the GPU run the hand-written HIP kernels (``csrc/hyper_dyt.hip``,
+``csrc/mlstm_scan.hip``, ``csrc/diff_attn.hip``) and a missing extension
+raises; CPU tensors run the torch implementations below, which are the
+CPU test tier's execution path.
+
+A step's batch is *ragged*: sequence b contributes ``new[b]`` tokens that
+continue ``pos0[b]`` cached ones. Tokens are flattened sequence after
+sequence; :class:`RaggedMeta` carries the offsets on the host and on the
+device, so a prompt portion and single decoded tokens of other requests
+share one forward pass.
+"""
+
+from __future__ import annotations
+
+from typing import List, Optional, Sequence
+
+import torch
+
+PAGE = 128
+
+
+class RaggedMeta:
+    """Flat-token description of one step.
+
+    ``new[b]`` tokens of sequence b start at flat offset ``cu[b]`` and at
+    position ``pos0[b]``; ``slots[b]`` is its state slot and ``table[b]``
+    its page-table row."""
+
+    def __init__(self, new: Sequence[int], pos0: Sequence[int],
+                 slots: Sequence[int], table: torch.Tensor, device):
+        assert len(new) == len(pos0) == len(slots) == table.shape[0]
+        self.new_h = [int(x) for x in new]
+        self.pos0_h = [int(x) for x in pos0]
+        self.slots_h = [int(x) for x in slots]
+        self.B = len(self.new_h)
+        cu = [0]
+        for x in self.new_h:
+            cu.append(cu[-1] + x)
+        self.cu_h = cu
+        self.T = cu[-1]
+        seq, pos = [], []
+        for b, (x, p) in enumerate(zip(self.new_h, self.pos0_h)):
+            seq += [b] * x
+            pos += range(p, p + x)
+        i32 = dict(dtype=torch.int32, device=device)
+        # ONE host->device copy for all the small index vectors
+        packed = torch.tensor(cu + self.slots_h + self.pos0_h + seq + pos,
+                              dtype=torch.int32).to(device)
+        B, T = self.B, self.T
+        self.cu = packed[:B + 1]
+        self.slots = packed[B + 1:2 * B + 1]
+        self.pos0 = packed[2 * B + 1:3 * B + 1]
+        self.tok_seq = packed[3 * B + 1:3 * B + 1 + T]
+        self.tok_pos = packed[3 * B + 1 + T:]
+        self.table = table.to(**i32).contiguous()
+        self.max_kv = max((p + x for p, x in zip(self.pos0_h, self.new_h)),
+                          default=0)
+
+    @property
+    def last_rows(self) -> List[int]:
+        """Flat index of every sequence's last token."""
+        return [c - 1 for c in self.cu_h[1:]]
+
+
+def _ext():
+    from tensorlink_amd import ops
+    return ops._require_ext()
+
+
+# ---------------------------------------------------------------------------
+# hyper-connections + Dynamic Tanh
+# ---------------------------------------------------------------------------
+def hyper_dyt(X: torch.Tensor, y: Optional[torch.Tensor] = None,
+              mix: Optional[torch.Tensor] = None,
+              out: Optional[torch.Tensor] = None,
+              inw: Optional[torch.Tensor] = None,
+              alpha: Optional[torch.Tensor] = None,
+              w: Optional[torch.Tensor] = None,
+              b: Optional[torch.Tensor] = None,
+              out_dtype=torch.float32, want_sum: bool = False):
+    """One pass over the fp32 residual streams X [ns, T, W] (in place).
+
+    If ``y`` is given, first X_t <- sum_s mix[s, t] X_s + out[t] * y. Then
+    u = sum_s inw[s] X_s (plain sum without ``inw``); returns
+    (tanh(alpha u) * w + b as ``out_dtype`` or None, u or None)."""
+    if X.is_cuda:
+        io32 = (y.dtype if y is not None else out_dtype) == torch.float32
+        h, u = _ext().hyper_dyt(X, y, mix, out, inw, alpha, w, b, io32,
+                                want_sum)
+        return (h if w is not None else None, u if want_sum else None)
+    if y is not None:
+        X.copy_(torch.einsum("st,sij->tij", mix, X)
+                + out.view(-1, 1, 1) * y.float())
+    u = X.sum(0) if inw is None else (inw.view(-1, 1, 1) * X).sum(0)
+    h = None
+    if w is not None:
+        h = (torch.tanh(alpha * u) * w + b).to(out_dtype)
+    return h, (u if want_sum else None)
+
+
+def relu_squared(x: torch.Tensor) -> torch.Tensor:
+    if x.is_cuda:
+        return _ext().relu_sq(x.contiguous())
+    return torch.relu(x) ** 2
+
+
+# ---------------------------------------------------------------------------
+# matrix memory
+# ---------------------------------------------------------------------------
+def soft_cap(x: torch.Tensor, cap: float) -> torch.Tensor:
+    return cap * torch.tanh(x / cap)
+
+
+def mlstm_scan(proj: torch.Tensor, offs, gates: torch.Tensor,
+               norm_w: torch.Tensor, S: torch.Tensor, n: torch.Tensor,
+               m: torch.Tensor, meta: RaggedMeta, H: int, D: int, V: int,
+               cap: float, eps: float) -> torch.Tensor:
+    """Stabilised matrix-memory recurrence for every sequence of the step.
+
+    proj [T, L] holds q | k | v | g at column offsets ``offs``; gates
+    [T, 2H] fp32 are the raw input | forget pre-activations. State pools
+    S [slots, H, D, V], n [slots, H, D], m [slots, H] (fp32) are read at
+    ``meta.slots`` (zero for a sequence with no cached tokens) and written
+    back. Returns [T, H*V]: per-head unit-RMS of the read-out, times
+    ``norm_w``, times sigmoid(g)."""
+    q_off, k_off, v_off, g_off = offs
+    qscale = D ** -0.5
+    if proj.is_cuda:
+        return _ext().mlstm_seq(proj, q_off, k_off, v_off, g_off,
+                                gates.contiguous(), norm_w, S, n, m,
+                                meta.cu, meta.slots, meta.pos0, H, D, V,
+                                cap, qscale, eps)
+    T = proj.shape[0]
+    pf = proj.float()
+    q = pf[:, q_off:q_off + H * D].view(T, H, D) * qscale
+    k = pf[:, k_off:k_off + H * D].view(T, H, D)
+    v = pf[:, v_off:v_off + H * V].view(T, H, V)
+    g = pf[:, g_off:g_off + H * V]
+    li = soft_cap(gates[:, :H], cap)
+    lf = torch.nn.functional.logsigmoid(soft_cap(gates[:, H:], cap))
+    o = torch.empty(T, H, V)
+    for b in range(meta.B):
+        slot = meta.slots_h[b]
+        if meta.pos0_h[b] == 0:
+            Sb = torch.zeros(H, D, V)
+            nb = torch.zeros(H, D)
+            mb = torch.zeros(H)
+        else:
+            Sb, nb, mb = S[slot].clone(), n[slot].clone(), m[slot].clone()
+        for t in range(meta.cu_h[b], meta.cu_h[b + 1]):
+            m_new = torch.maximum(lf[t] + mb, li[t])
+            a = torch.exp(lf[t] + mb - m_new)
+            bb = torch.exp(li[t] - m_new)
+            Sb = a[:, None, None] * Sb + bb[:, None, None] * (
+                k[t].unsqueeze(-1) * v[t].unsqueeze(-2))
+            nb = a[:, None] * nb + bb[:, None] * k[t]
+            mb = m_new
+            num = (Sb * q[t].unsqueeze(-1)).sum(1)
+            den = torch.maximum((nb * q[t]).sum(-1).abs(),
+                                torch.exp(-mb)) + 1e-6
+            o[t] = num / den[:, None]
+        if meta.new_h[b] > 0:
+            S[slot], n[slot], m[slot] = Sb, nb, mb
+    o = o * torch.rsqrt((o * o).mean(-1, keepdim=True) + eps)
+    out = o.reshape(T, H * V) * norm_w * torch.sigmoid(g)
+    return out.to(proj.dtype)
+
+
+# ---------------------------------------------------------------------------
+# differential attention over the paged pool
+# ---------------------------------------------------------------------------
+def kv_append(proj: torch.Tensor, k_off: int, v_off: int,
+              kpool: torch.Tensor, vpool: torch.Tensor,
+              meta: RaggedMeta) -> None:
+    """Write the step's key rows [G*DK] and value rows [G*V] (columns
+    ``k_off`` / ``v_off`` of proj) into pools [pages, G, PAGE, *]."""
+    if proj.is_cuda:
+        _ext().kv_append(proj, k_off, v_off, kpool, vpool, meta.tok_seq,
+                         meta.tok_pos, meta.table)
+        return
+    G, DK, V = kpool.shape[1], kpool.shape[3], vpool.shape[3]
+    T = proj.shape[0]
+    pos = meta.tok_pos.long()
+    page = meta.table.long()[meta.tok_seq.long(), pos // PAGE]
+    r = pos % PAGE
+    kpool[page, :, r] = proj[:, k_off:k_off + G * DK].view(T, G, DK)
+    vpool[page, :, r] = proj[:, v_off:v_off + G * V].view(T, G, V)
+
+
+def diff_attention(q: torch.Tensor, q_off: int, kpool: torch.Tensor,
+                   vpool: torch.Tensor, meta: RaggedMeta, lam: torch.Tensor,
+                   H: int, D: int, scale: float, diff: float,
+                   eps: float) -> torch.Tensor:
+    """Two-map attention of the step's tokens over their sequences' cached
+    keys/values (the step's own rows already appended). Query rows are
+    [H, 2, D] at column ``q_off``; returns [T, H*V] =
+    unit_rms(a1 - lam * a2) * (1 - diff) per head."""
+    if q.is_cuda:
+        return _ext().diff_attn_rows(q, q_off, kpool, vpool, meta.tok_seq,
+                                     meta.tok_pos, meta.table, lam, H, D,
+                                     scale, diff, eps)
+    G, V = kpool.shape[1], vpool.shape[3]
+    T = q.shape[0]
+    out = torch.empty(T, H, V)
+    qf = q[:, q_off:q_off + H * 2 * D].float().view(T, H, 2, D)
+    rep = H // G
+    for b in range(meta.B):
+        t0, t1 = meta.cu_h[b], meta.cu_h[b + 1]
+        if t1 == t0:
+            continue
+        L = meta.pos0_h[b] + (t1 - t0)
+        pages = meta.table[b, :(L + PAGE - 1) // PAGE].long()
+        # [L, G, *]
+        kb = kpool[pages].float().permute(0, 2, 1, 3).reshape(
+            -1, G, 2, D)[:L]
+        vb = vpool[pages].float().permute(0, 2, 1, 3).reshape(-1, G, V)[:L]
+        kb = kb.repeat_interleave(rep, 1)                  # [L, H, 2, D]
+        vb = vb.repeat_interleave(rep, 1)
+        sc = torch.einsum("thmd,jhmd->hmtj", qf[t0:t1], kb) * scale
+        qpos = torch.arange(meta.pos0_h[b], L).view(-1, 1)
+        mask = torch.arange(L).view(1, -1) > qpos
+        sc = sc.masked_fill(mask, float("-inf"))
+        a = torch.einsum("hmtj,jhv->mthv", torch.softmax(sc, -1), vb)
+        out[t0:t1] = a[0] - lam.float() * a[1]
+    out = out * torch.rsqrt((out * out).mean(-1, keepdim=True) + eps)
+    return (out * (1.0 - diff)).reshape(T, H * V).to(q.dtype)
+
+
+# ---------------------------------------------------------------------------
+# routing
+# ---------------------------------------------------------------------------
+def group_limited_router(logits: torch.Tensor, top: int, n_groups: int,
+                         keep_groups: int, scale: float):
+    """Softmax scores over all experts; experts form ``n_groups`` equal
+    groups of neighbours scored by their best member, and only the
+    ``keep_groups`` best groups stay eligible. The ``top`` best eligible
+    experts are chosen; weights = their scores / (sum + 1e-20) * scale.
+
+    logits [T, E] fp32 -> (weights [T, top] fp32, indices [T, top])."""
+    s = torch.softmax(logits.float(), -1)
+    T, E = s.shape
+    if keep_groups < n_groups:
+        gs = s.view(T, n_groups, E // n_groups).amax(-1)
+        kept = gs.topk(keep_groups, dim=-1).indices
+        allow = torch.zeros(T, n_groups, dtype=torch.bool, device=s.device)
+        allow.scatter_(1, kept, True)
+        allow = allow.unsqueeze(-1).expand(T, n_groups, E // n_groups)
+        masked = s.masked_fill(~allow.reshape(T, E), -1.0)
+    else:
+        masked = s
+    idx = masked.topk(top, dim=-1).indices
+    w = s.gather(1, idx)
+    w = w / (w.sum(-1, keepdim=True) + 1e-20) * scale
+    return w, idx

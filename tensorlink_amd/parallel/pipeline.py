@@ -98,7 +98,9 @@ class PipelineRunner:
         import os as _os
         self.kv_mode = kv_mode or _os.environ.get("TL_KV_MODE",
                                                   "contiguous")
-        self._no_graph = False
+        # stages that build host-side batch metadata every step opt out
+        # of hipGraph-captured decode
+        self._no_graph = not getattr(self.stage, "GRAPH_CAPTURE", True)
         if quantize == "fp8":
             from tensorlink_amd import ops as _ops
             from tensorlink_amd.models.quant import quantize_experts_fp8
