@@ -91,6 +91,12 @@ class _SlotView:
         self.batch = len(slot_ids)
         self.pages_per_seq = cache.pages_per_seq
         self._parent = cache
+        # layered models: which state slot each row uses, the per-layer
+        # recurrent state, and (set by the ragged path) the flat-batch
+        # description of the step
+        self.slot_ids = list(slot_ids)
+        self.state = getattr(cache, "state", None)
+        self.ragged = None
 
     def advance(self, n):
         pass   # slot lengths are tracked by the scheduler
@@ -136,9 +142,24 @@ class ContinuousBatcher:
         self.spec_k = spec_k
         self.slot_ctx: List[Optional[list]] = [None] * max_slots
         self.spec_accepted = 0
-        self.cache = cache_cls(
-            self.stage.num_layers, max_slots, pool_pages, max_ctx,
-            self.stage.config, runner.device, runner.dtype)
+        # a stage that serves a mixed ragged batch in one forward (prompt
+        # portions beside single decoded tokens) gets ONE model call per
+        # scheduler iteration instead of a prefill call plus a decode call
+        self.ragged = bool(getattr(self.stage, "SUPPORTS_RAGGED", False))
+        if hasattr(self.stage, "make_slot_cache"):
+            # layered models own their cache layout (per-layer head sizes,
+            # shared KV, recurrent state slots)
+            if prefix_caching or speculative:
+                raise ValueError(
+                    "prefix caching / speculation need a pure KV cache; "
+                    "this model keeps recurrent state per slot")
+            self.cache = self.stage.make_slot_cache(
+                max_slots, pool_pages, max_ctx, runner.device, runner.dtype)
+        else:
+            self.cache = cache_cls(
+                self.stage.num_layers, max_slots, pool_pages, max_ctx,
+                self.stage.config, runner.device, runner.dtype)
+        self._forced = {}                 # request id -> slot (forced_step)
         self.max_slots = max_slots
         self.prefill_chunk = prefill_chunk    # None = whole prompt at once
         self.slots: List[Optional[Request]] = [None] * max_slots
@@ -230,6 +251,8 @@ class ContinuousBatcher:
         the resume path when pages free up. vLLM-style preemption keeps
         admission live when the page pool starves."""
         from tensorlink_amd.models.paged import swap_out
+        if not getattr(self.cache, "SWAPPABLE", True):
+            return False
         cands = [i for i, r in enumerate(self.slots)
                  if r is not None and not self._prefilling(i)
                  and self.slot_filled[i] > 0 and i != exclude]
@@ -512,6 +535,158 @@ class ContinuousBatcher:
         self.steps += 1
         return True
 
+    # ---------------- ragged (single-forward) path --------------------
+    @torch.no_grad()
+    def _forward_ragged(self, items, lookahead: int = 1):
+        """Run ONE forward over ``items`` = [(slot, start, token ids)]:
+        each slot contributes its tokens at positions start.. on top of
+        what its pages and state slot already hold. Returns the stage's
+        pre-head output [T, H] and the step's RaggedMeta."""
+        from tensorlink_amd.ops.mixers import RaggedMeta
+        for slot, start, toks in items:
+            need = start + len(toks) + lookahead
+            try:
+                self.cache.ensure(slot, need)
+            except RuntimeError:
+                if not self._preempt_one(exclude=slot):
+                    raise
+                self.cache.ensure(slot, need)
+        slot_ids = [it[0] for it in items]
+        meta = RaggedMeta([len(it[2]) for it in items],
+                          [it[1] for it in items], slot_ids,
+                          self.cache.table[slot_ids], self.device)
+        view = _SlotView(self.cache, slot_ids, meta.pos0)
+        view.ragged = meta
+        flat = [t for it in items for t in it[2]]
+        ids = torch.tensor(flat, device=self.device,
+                           dtype=torch.int64).unsqueeze(0)
+        hidden = self.stage(ids, meta.tok_pos.unsqueeze(0), kv_cache=view,
+                            return_logits=False)
+        return hidden[0], meta
+
+    @torch.no_grad()
+    def _ragged_iteration(self) -> bool:
+        """One scheduler iteration as a single model call: the next
+        portion of ONE prefilling slot beside one token of every decoding
+        slot. Sampling and retirement follow the two-call path."""
+        items, kinds = [], []
+        pre_slot = None
+        for slot in range(self.max_slots):
+            req = self.slots[slot]
+            if req is None or not (self._prefilling(slot)
+                                   or self.slot_filled[slot] == 0):
+                continue
+            if req.cancelled:
+                req.tokens.put(None)
+                req.done.set()
+                self.slots[slot] = None
+                self.slot_prompt[slot] = None
+                self.cache.release_slot(slot)
+                continue
+            prompt = self.slot_prompt[slot]
+            total = prompt.numel()
+            start = self.slot_filled[slot]
+            end = (total if self.prefill_chunk is None
+                   else min(start + self.prefill_chunk, total))
+            items.append((slot, start, prompt[start:end].tolist()))
+            kinds.append(("prefill", end, total))
+            pre_slot = slot
+            break
+        for i, req in enumerate(self.slots):
+            if (req is None or i == pre_slot or self._prefilling(i)
+                    or self.slot_filled[i] == 0):
+                continue
+            items.append((i, self.slot_len[i], [self.slot_last[i]]))
+            kinds.append(("decode", None, None))
+        if not items:
+            return False
+        try:
+            hidden, meta = self._forward_ragged(items)
+        except Exception as e:
+            if pre_slot is None:
+                raise
+            req = self.slots[pre_slot]      # fail the joining request only
+            req.error = str(e)
+            req.tokens.put(None)
+            req.done.set()
+            self.slots[pre_slot] = None
+            self.slot_prompt[pre_slot] = None
+            self.cache.release_slot(pre_slot)
+            return True
+        last = meta.last_rows
+        pick = [k for k, kd in enumerate(kinds)
+                if kd[0] == "decode" or kd[1] == kd[2]]
+        for k, kd in enumerate(kinds):
+            if kd[0] == "prefill":
+                self.slot_filled[items[k][0]] = kd[1]
+        if pick:
+            rows = hidden[torch.tensor([last[k] for k in pick],
+                                       device=hidden.device)]
+            logits = self.stage.head(rows)
+            slots = [items[k][0] for k in pick]
+            toks = self._sample(logits, [self.slots[i] for i in slots],
+                                slots=slots)
+            for k, i, tok in zip(pick, slots, toks):
+                req = self.slots[i]
+                if kinds[k][0] == "prefill":
+                    self.slot_len[i] = kinds[k][2]
+                    self.slot_emitted[i] = 1
+                else:
+                    self.slot_len[i] += 1
+                    self.slot_emitted[i] += 1
+                self.slot_last[i] = tok
+                self.slot_counts[i][tok] = \
+                    self.slot_counts[i].get(tok, 0) + 1
+                req.tokens.put(tok)
+                self._maybe_finish(i, tok)
+        self.steps += 1
+        return True
+
+    @torch.no_grad()
+    def forced_step(self, entries, end=()):
+        """Teacher-forced step for trace replay and scoring: ``entries`` =
+        [(request id, next token ids, offsets among them whose logits are
+        wanted)]. All entries run as one ragged batch on the scheduler's
+        own slots, pages and state; a request takes a free slot at its
+        first entry and gives slot and pages back when named in ``end``.
+        Returns fp32 logits [n_wanted, vocab] on the host (None if nothing
+        is wanted). Not to be mixed with a running scheduler thread."""
+        assert self.ragged, "forced_step needs a ragged-capable stage"
+        assert self._thread is None, "scheduler thread is running"
+        items, wants = [], []
+        for rid, toks, want in entries:
+            if not len(toks):
+                continue
+            slot = self._forced.get(rid)
+            if slot is None:
+                slot = self._free_slot()
+                if slot is None:
+                    raise RuntimeError("no free slot for request %r" % rid)
+                self._forced[rid] = slot
+                self.slots[slot] = Request(
+                    input_ids=torch.empty(0, dtype=torch.int64))
+                self.slot_len[slot] = 0
+            items.append((slot, self.slot_len[slot], list(toks)))
+            wants.append(list(want))
+        out = None
+        if items:
+            hidden, meta = self._forward_ragged(items, lookahead=0)
+            rows = [meta.cu_h[b] + w for b, ws in enumerate(wants)
+                    for w in ws]
+            if rows:
+                sel = hidden[torch.tensor(rows, device=hidden.device)]
+                out = self.stage.head(sel).float().cpu()
+            for slot, _, toks in items:
+                self.slot_len[slot] += len(toks)
+        for rid in end:
+            slot = self._forced.pop(rid, None)
+            if slot is not None:
+                self.slots[slot] = None
+                self.slot_len[slot] = 0
+                self.cache.release_slot(slot)
+        self.steps += 1
+        return out
+
     def _loop(self):
         self._drain = False
         while not self._stop.is_set() or (
@@ -567,6 +742,13 @@ class ContinuousBatcher:
                     self.slot_filled[slot] = self.cache.adopt_prefix(
                         slot, req.input_ids.tolist())
                 admitted = True
+            if self.ragged:
+                # prompt portion + decode rows in ONE forward
+                busy = self._ragged_iteration()
+                if not busy and not admitted:
+                    self._wake.wait(0.05)
+                    self._wake.clear()
+                continue
             # one prefill chunk per iteration: bounds how long running
             # decodes wait behind a new long prompt
             prefilled = False
