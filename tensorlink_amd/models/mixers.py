@@ -16,6 +16,7 @@ expert GEMMs run in the serving dtype with fp32 accumulation.
 
 from __future__ import annotations
 
+import os
 from typing import Optional
 
 import torch
@@ -184,7 +185,8 @@ class GroupLimitedMoE(nn.Module, _F32Cache):
     def _grouped_ok(self, h) -> bool:
         return (h.is_cuda and h.dtype == torch.bfloat16
                 and ops.extension_loaded()
-                and self.W % 64 == 0 and self.ff % 64 == 0)
+                and self.W % 64 == 0 and self.ff % 64 == 0
+                and not os.environ.get("TL_NO_GROUPED_MOE"))
 
     def _tables(self, dev):
         key = (self.up.data_ptr(), self.down.data_ptr(), str(dev))

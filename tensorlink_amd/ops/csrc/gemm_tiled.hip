@@ -56,7 +56,7 @@ __global__ __launch_bounds__(BLOCK, 2) void gemm_tiled_kernel(
   const int m_base = blockIdx.z * (MT * 16);
 
   const int split = SPLIT ? blockIdx.y : 0;
-  const int k_per = SPLIT ? ((K / 64 + n_split - 1) / n_split) * 64 : K;
+  const int k_per = SPLIT ? (((K + 63) / 64 + n_split - 1) / n_split) * 64 : K;
   const int k_begin = split * k_per;
   const int k_end = min(K, k_begin + k_per);
 
@@ -208,7 +208,7 @@ __global__ __launch_bounds__(512, 1) void gemm_tiled_sq_kernel(
   const int m_base = blockIdx.z * 256;
 
   const int split = SPLIT ? blockIdx.y : 0;
-  const int k_per = SPLIT ? ((K / 64 + n_split - 1) / n_split) * 64 : K;
+  const int k_per = SPLIT ? (((K + 63) / 64 + n_split - 1) / n_split) * 64 : K;
   const int k_begin = split * k_per;
   const int k_end = min(K, k_begin + k_per);
 

@@ -289,6 +289,9 @@ def test_decode_attn_mfma(B, Hq, Hkv, D, L, ns):
     (16, 3584, 3584, False),      # small-batch decode (streaming)
     (7, 1024, 256, True),         # tiny M, M tail
     (33, 512, 96, False),         # K%64==32 tail path
+    (23, 256, 288, False),        # K%64==32 tail under split-K (streaming)
+    (100, 256, 288, True),        # K%64==32 tail under split-K (tiled)
+    (439, 448, 352, False),       # same, several m-blocks
 ])
 @torch.no_grad()
 def test_tl_gemm(M, N, K, bias):
