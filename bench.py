@@ -43,7 +43,12 @@ def parse_args():
     p.add_argument("--new-tokens", type=int, default=128)
     p.add_argument("--micro-batches", type=int, default=0,
                    help="decode micro-batches in flight (0 => world size)")
-    p.add_argument("--mode", choices=["serve", "train"], default="serve")
+    p.add_argument("--mode", choices=["serve", "train", "layered"],
+                   default="serve",
+                   help="layered: Kepusun-family prefill/decode throughput "
+                        "beside an equal-size Qwen3-MoE-shaped model")
+    p.add_argument("--sizes", default="w1024,w2048",
+                   help="layered mode: comma list of size presets")
     p.add_argument("--dp", type=int, default=1,
                    help="data-parallel replicas (train mode; world=dp*pp)")
     return p.parse_args()
@@ -97,6 +102,111 @@ def run_train(args, rank, world, device, use_gpu, config):
         }))
 
 
+LAYERED_SIZES = {
+    # width, layers are [mlstm, attention, mlstm, attention(shared KV)]
+    "w1024": dict(width=1024, heads=8, kv=2, dim=64, vdim=128, experts=16,
+                  top=2, ff=512, vocab=32000, batch=8, prompt=2048),
+    "w2048": dict(width=2048, heads=16, kv=4, dim=64, vdim=128, experts=32,
+                  top=4, ff=768, vocab=32000, batch=8, prompt=2048),
+    "tiny": dict(width=128, heads=2, kv=1, dim=32, vdim=64, experts=4,
+                 top=2, ff=64, vocab=512, batch=2, prompt=96),
+}
+
+
+def layered_configs(z):
+    """(Kepusun config, equal-size Qwen3-MoE-shaped config) of a preset:
+    same width, depth, vocabulary, expert count/top/width; the attention
+    model gets heads * head_dim equal to the mixers' value width."""
+    from tensorlink_amd.models.configs import ModelConfig
+    from tensorlink_amd.models.kepusun import KepusunConfig
+    mlp = {"kind": "moe", "expert": {"ff": z["ff"]},
+           "router": {"experts": z["experts"], "top": z["top"],
+                      "scale": 1.0,
+                      "groups": {"count": 4, "keep": 2}}}
+    ml = {"type": "mlstm", "mlp": mlp,
+          "mixer": {"heads": z["heads"], "dim": z["dim"],
+                    "vdim": z["vdim"], "gate_cap": 15.0}}
+    at = {"heads": z["heads"], "kv_heads": z["kv"], "dim": z["dim"],
+          "vdim": z["vdim"], "scale": z["dim"] ** -0.5, "diff": 0.5}
+    layers = [ml, {"type": "attention", "mlp": mlp, "mixer": at}, ml,
+              {"type": "attention", "mlp": mlp,
+               "mixer": dict(at, kv_from=1)}]
+    kep = KepusunConfig.from_dict({
+        "architecture": "Kepusun", "vocab": z["vocab"],
+        "width": z["width"], "streams": 2, "norm": {"eps": 1e-6},
+        "layers": layers}, name="kepusun-" + str(z["width"]))
+    ref = ModelConfig(
+        name="qwen3-moe-" + str(z["width"]), vocab_size=z["vocab"],
+        hidden_size=z["width"], intermediate_size=z["ff"] * z["experts"],
+        num_hidden_layers=len(layers), num_attention_heads=z["heads"],
+        num_key_value_heads=z["kv"], head_dim=z["vdim"],
+        max_position_embeddings=8192, num_local_experts=z["experts"],
+        num_experts_per_tok=z["top"], expert_intermediate_size=z["ff"],
+        architecture="qwen3")
+    return kep, ref
+
+
+@torch.no_grad()
+def run_layered(args, device, use_gpu):
+    """Prefill and decode tokens/s of the Kepusun family beside the
+    closest existing family at equal size; one JSON line per preset."""
+    dtype = torch.bfloat16 if use_gpu else torch.float32
+    new = min(args.new_tokens, 32)
+
+    def sync():
+        if use_gpu:
+            torch.cuda.synchronize()
+
+    def measure(config, B, S):
+        plan = plan_for_world(config, 1, batch_size=B, seq_len=S + new + 1)
+        runner = PipelineRunner(plan, 0, 1, device=device, init="random",
+                                seed=7, dtype=dtype)
+        stage = runner.stage
+        torch.manual_seed(3)
+        ids = torch.randint(0, config.vocab_size, (B, S), device=device)
+        pos = torch.arange(S, device=device,
+                           dtype=torch.int32).unsqueeze(0).repeat(B, 1)
+        out = {}
+        for it in range(args.warmup + args.steps):
+            if it == args.warmup:
+                t_pre = t_dec = 0.0
+            cache = runner.alloc_cache(B, S + new + 1)
+            sync()
+            t0 = time.perf_counter()
+            hidden = stage(ids, pos, kv_cache=cache, return_logits=False)
+            cur = stage.head(hidden[:, -1:]).argmax(-1)
+            sync()
+            t1 = time.perf_counter()
+            p = torch.full((B, 1), S, device=device, dtype=torch.int32)
+            for _ in range(new):
+                cur = stage(cur, p, kv_cache=cache).argmax(-1)
+                p = p + 1
+            sync()
+            t2 = time.perf_counter()
+            if it >= args.warmup:
+                t_pre += t1 - t0
+                t_dec += t2 - t1
+        out["prefill_tokens_per_s"] = B * S * args.steps / t_pre
+        out["decode_tokens_per_s"] = B * new * args.steps / t_dec
+        out["params_m"] = config.param_count() / 1e6
+        del runner
+        if use_gpu:
+            torch.cuda.empty_cache()
+        return out
+
+    for name in args.sizes.split(","):
+        z = LAYERED_SIZES[name]
+        kep, ref = layered_configs(z)
+        B, S = z["batch"], z["prompt"]
+        res = {"kepusun": measure(kep, B, S), "qwen3_moe": measure(ref, B, S)}
+        print(json.dumps({
+            "metric": "layered-family prefill/decode tokens/sec",
+            "size": name, "batch": B, "prompt_len": S, "new_tokens": new,
+            "steps": args.steps, "warmup": args.warmup,
+            "dtype": "bf16" if use_gpu else "fp32", "data": "synthetic",
+            **res}))
+
+
 def main():
     args = parse_args()
     rank, world = init_distributed()
@@ -115,6 +225,10 @@ def main():
     from tensorlink_amd.utils.tunable import setup_tunableop
     setup_tunableop(tune=bool(os.environ.get("TL_TUNE")))
 
+    if args.mode == "layered":
+        assert world == 1, "layered mode is a single-GPU comparison"
+        run_layered(args, device, use_gpu)
+        return
     config = get_config(args.model)
     if args.mode == "train":
         run_train(args, rank, world, device, use_gpu, config)

@@ -178,6 +178,7 @@ class KepusunStageModel(nn.Module):
                                      dtype)
         for s in range(batch):
             cache.ensure(s, max_seq)
+        cache.static = True
         return cache
 
     # -------------------------------------------------------- forward

@@ -199,6 +199,13 @@ class HybridSlotCache(DynamicPagedKVCache):
                                  dtype=torch.int32)
         self._slot_pages = [[] for _ in range(slots)]
         self.slot_ids = list(range(slots))
+        self.static = False     # True: every slot keeps its pages on reset
+
+    def reset(self):
+        if self.static:
+            self.seq_lens.zero_()
+        else:
+            super().reset()
 
     def slice(self, s: int, e: int):
         """View over slots s..e-1 (micro-batch split of a rectangular

@@ -31,6 +31,11 @@ int tl_diff_attn_rows(const void* q, int ldq, int q_off, const void* kpool,
                       const void* lam, void* out, int T, int H, int G, int D,
                       int V, float scale, float diff, float eps, int is_f32,
                       hipStream_t stream);
+int tl_diff_attn_tiles(const void* q, int ldq, int q_off, const void* kpool,
+                       const void* vpool, const void* tiles, int n_tiles,
+                       const void* table, int P, const void* lam, void* out,
+                       int H, int G, int D, int V, float scale, float diff,
+                       float eps, hipStream_t stream);
 }
 
 namespace {
@@ -225,6 +230,43 @@ Tensor diff_attn_rows(Tensor q, int64_t q_off, Tensor kpool, Tensor vpool,
   return out;
 }
 
+// MFMA path for prompt portions (bf16): `tiles` [n, 4] int32 rows of
+// (sequence, first flat token, token count <= 64, first position).
+// Returns false when the shape is outside the kernel's range.
+bool diff_attn_tiles(Tensor q, int64_t q_off, Tensor kpool, Tensor vpool,
+                     Tensor tiles, Tensor table, Tensor lam, Tensor out,
+                     int64_t H, int64_t D, double scale, double diff,
+                     double eps) {
+  MIX_IN(q);
+  MIX_IN(kpool);
+  MIX_IN(vpool);
+  MIX_IN(out);
+  MIX_I32(tiles);
+  MIX_I32(table);
+  MIX_F32(lam);
+  TORCH_CHECK(q.scalar_type() == torch::kBFloat16 &&
+                  kpool.scalar_type() == torch::kBFloat16 &&
+                  vpool.scalar_type() == torch::kBFloat16 &&
+                  out.scalar_type() == torch::kBFloat16,
+              "the tiled kernel is bf16 only");
+  TORCH_CHECK(kpool.dim() == 4 && vpool.dim() == 4 && kpool.size(2) == 128 &&
+                  vpool.size(2) == 128 && kpool.size(1) == vpool.size(1) &&
+                  kpool.size(3) == 2 * D,
+              "pools must be [pages, G, 128, 2D] / [pages, G, 128, V]");
+  const int64_t T = q.size(0), ld = q.size(1);
+  const int G = kpool.size(1), V = vpool.size(3);
+  TORCH_CHECK(q_off + H * 2 * D <= ld, "query columns out of range");
+  TORCH_CHECK(tiles.dim() == 2 && tiles.size(1) == 4 && table.dim() == 2,
+              "tiles must be [n, 4]");
+  TORCH_CHECK(out.numel() == T * H * V, "out must be [T, H*V]");
+  const int rc = tl_diff_attn_tiles(
+      q.data_ptr(), (int)ld, (int)q_off, kpool.data_ptr(), vpool.data_ptr(),
+      tiles.data_ptr(), (int)tiles.size(0), table.data_ptr(),
+      (int)table.size(1), lam.data_ptr(), out.data_ptr(), (int)H, G, (int)D,
+      V, (float)scale, (float)diff, (float)eps, mix_stream());
+  return rc == 0;
+}
+
 }  // namespace
 
 void register_mix_ops(pybind11::module& mod) {
@@ -234,6 +276,8 @@ void register_mix_ops(pybind11::module& mod) {
   mod.def("mlstm_seq", &mlstm_seq,
           "matrix-memory recurrence over ragged sequences (slot state)");
   mod.def("kv_append", &kv_append, "scatter new K/V rows into page pools");
+  mod.def("diff_attn_tiles", &diff_attn_tiles,
+          "differential attention on MFMA, 64-query tiles, paged KV (bf16)");
   mod.def("diff_attn_rows", &diff_attn_rows,
           "differential attention, one query token per block, paged KV");
 }

@@ -34,8 +34,12 @@ DEVINLINE float log_sigmoid(float x) {
   return fminf(x, 0.f) - log1pf(expf(-fabsf(x)));
 }
 
-template <typename T, int DMAX>
-__global__ void mlstm_seq_kernel(
+// TB tokens are staged per round: their q/k rows and capped gates go to
+// LDS in one sweep (one global-memory latency per round instead of one per
+// token), v and the output gate wait in registers, and the per-token
+// normaliser / RMS reductions of the whole round share one barrier.
+template <typename T, int DMAX, int TB, int NTMAX>
+__global__ __launch_bounds__(NTMAX) void mlstm_seq_kernel(
     const T* __restrict__ proj, int ld, int q_off, int k_off, int v_off,
     int g_off,
     const float* __restrict__ gates,   // [Ttot, 2H] raw (input | forget)
@@ -49,12 +53,16 @@ __global__ void mlstm_seq_kernel(
   extern __shared__ float lds[];
   const int h = blockIdx.x, b = blockIdx.y;
   const int c = threadIdx.x;
-  const int nw = blockDim.x / WAVE_SIZE;
+  const int nt = blockDim.x;
+  const int nw = nt / WAVE_SIZE;
   const int lane = c & (WAVE_SIZE - 1), wave = c / WAVE_SIZE;
-  // lds: q[2][D] | k[2][D] | red[2][nw + 1]
+  // lds: q[TB][D] | k[TB][D] | li[TB] | lf[TB] | nq[TB] | red[TB][nw]
   float* lq = lds;
-  float* lk = lds + 2 * D;
-  float* red = lds + 4 * D;
+  float* lk = lq + TB * D;
+  float* lli = lk + TB * D;
+  float* llf = lli + TB;
+  float* lnq = llf + TB;
+  float* red = lnq + TB;
 
   const int t0 = cu[b], t1 = cu[b + 1];
   if (t0 >= t1) return;
@@ -75,52 +83,84 @@ __global__ void mlstm_seq_kernel(
     s[d] = v;
   }
   float m = fresh ? 0.f : m_pool[(int64_t)slot * H + h];
+  const float nw_c = is_col ? norm_w[h * V + c] : 0.f;
 
-  for (int t = t0; t < t1; ++t) {
-    const int par = (t - t0) & 1;
-    const T* row = proj + (int64_t)t * ld;
-    for (int d = c; d < D; d += blockDim.x) {
-      lq[par * D + d] = ldv<T>(row + q_off + h * D + d) * qscale;
-      lk[par * D + d] = ldv<T>(row + k_off + h * D + d);
+  for (int tb0 = t0; tb0 < t1; tb0 += TB) {
+    const int cnt = min(TB, t1 - tb0);
+    // ---- stage the round
+    for (int i = c; i < cnt * D; i += nt) {
+      const int tt = i / D, d = i - tt * D;
+      const T* row = proj + (int64_t)(tb0 + tt) * ld;
+      lq[tt * D + d] = ldv<T>(row + q_off + h * D + d) * qscale;
+      lk[tt * D + d] = ldv<T>(row + k_off + h * D + d);
     }
-    const float gi = gates[(int64_t)t * 2 * H + h];
-    const float gf = gates[(int64_t)t * 2 * H + H + h];
-    const float li = cap * tanhf(gi / cap);
-    const float lf = log_sigmoid(cap * tanhf(gf / cap));
-    const float m_new = fmaxf(lf + m, li);
-    const float a = expf(lf + m - m_new);
-    const float bb = expf(li - m_new);
-    m = m_new;
-    const float vc = is_col ? ldv<T>(row + v_off + h * V + c)
-                            : (is_n ? 1.f : 0.f);
-    __syncthreads();
-    float num = 0.f;
-    const float bv = bb * vc;
-    const float* qq = lq + par * D;
-    const float* kk = lk + par * D;
+    if (c < cnt) {
+      const float gi = gates[(int64_t)(tb0 + c) * 2 * H + h];
+      const float gf = gates[(int64_t)(tb0 + c) * 2 * H + H + h];
+      lli[c] = cap * tanhf(gi / cap);
+      llf[c] = log_sigmoid(cap * tanhf(gf / cap));
+    }
+    float vreg[TB], greg[TB], num[TB], em[TB];
 #pragma unroll
-    for (int d = 0; d < DMAX; ++d) {
-      if (d < D) {
-        s[d] = a * s[d] + bv * kk[d];
-        num += s[d] * qq[d];
+    for (int tt = 0; tt < TB; ++tt) {
+      vreg[tt] = is_n ? 1.f : 0.f;
+      greg[tt] = 0.f;
+      if (tt < cnt && is_col) {
+        const T* row = proj + (int64_t)(tb0 + tt) * ld;
+        vreg[tt] = ldv<T>(row + v_off + h * V + c);
+        greg[tt] = ldv<T>(row + g_off + h * V + c);
       }
     }
-    const float sq = wave_reduce_sum(is_col ? num * num : 0.f);
-    float* rr = red + par * (nw + 1);
-    if (lane == 0) rr[wave] = sq;
-    if (is_n) rr[nw] = num;
     __syncthreads();
-    float ss = 0.f;
-    for (int w = 0; w < nw; ++w) ss += rr[w];
-    const float den = fmaxf(fabsf(rr[nw]), expf(-m)) + 1e-6f;
-    if (is_col) {
-      const float o = num / den;
-      const float r = rsqrtf(ss / (den * den) / (float)V + eps);
-      const float g = ldv<T>(row + g_off + h * V + c);
-      const float sg = 1.f / (1.f + expf(-g));
-      stv<T>(out + (int64_t)t * H * V + h * V + c,
-             o * r * norm_w[h * V + c] * sg);
+    // ---- the recurrence, token by token, no barrier inside
+#pragma unroll
+    for (int tt = 0; tt < TB; ++tt) {
+      num[tt] = 0.f;
+      em[tt] = 0.f;
+      if (tt < cnt) {
+        const float li = lli[tt], lf = llf[tt];
+        const float m_new = fmaxf(lf + m, li);
+        const float a = expf(lf + m - m_new);
+        const float bv = expf(li - m_new) * vreg[tt];
+        m = m_new;
+        em[tt] = expf(-m_new);
+        const float* qq = lq + tt * D;
+        const float* kk = lk + tt * D;
+        float acc = 0.f;
+#pragma unroll
+        for (int d = 0; d < DMAX; ++d) {
+          if (d < D) {
+            s[d] = a * s[d] + bv * kk[d];
+            acc += s[d] * qq[d];
+          }
+        }
+        num[tt] = acc;
+      }
     }
+    // ---- reductions of the whole round behind one barrier
+#pragma unroll
+    for (int tt = 0; tt < TB; ++tt) {
+      const float sq = wave_reduce_sum(is_col ? num[tt] * num[tt] : 0.f);
+      if (lane == 0) red[tt * nw + wave] = sq;
+      if (is_n) lnq[tt] = num[tt];
+    }
+    __syncthreads();
+    if (is_col) {
+#pragma unroll
+      for (int tt = 0; tt < TB; ++tt) {
+        if (tt < cnt) {
+          float ss = 0.f;
+          for (int w = 0; w < nw; ++w) ss += red[tt * nw + w];
+          const float den = fmaxf(fabsf(lnq[tt]), em[tt]) + 1e-6f;
+          const float o = num[tt] / den;
+          const float r = rsqrtf(ss / (den * den) / (float)V + eps);
+          const float sg = 1.f / (1.f + expf(-greg[tt]));
+          stv<T>(out + (int64_t)(tb0 + tt) * H * V + h * V + c,
+                 o * r * nw_c * sg);
+        }
+      }
+    }
+    __syncthreads();     // red / lq / lk are rewritten by the next round
   }
 #pragma unroll
   for (int d = 0; d < DMAX; ++d) {
@@ -146,21 +186,28 @@ int tl_mlstm_seq(const void* proj, int ld, int q_off, int k_off, int v_off,
   if (D > 256 || V + 1 > 1024 || B < 1) return 1;
   const int nt = ((V + 1 + WAVE_SIZE - 1) / WAVE_SIZE) * WAVE_SIZE;
   const int nw = nt / WAVE_SIZE;
-  const size_t smem = sizeof(float) * (4 * D + 2 * (nw + 1));
   dim3 grid(H, B), block(nt);
-#define TL_ML_LAUNCH(TT, DM)                                                 \
-  hipLaunchKernelGGL((mlstm_seq_kernel<TT, DM>), grid, block, smem, stream,  \
-                     (const TT*)proj, ld, q_off, k_off, v_off, g_off,        \
-                     (const float*)gates, (const float*)norm_w, (float*)S,   \
-                     (float*)n, (float*)m, (const int*)cu,                   \
-                     (const int*)slots, (const int*)pos0, (TT*)out, H, D, V, \
-                     cap, qscale, eps)
-#define TL_ML_D(TT)                                  \
-  if (D <= 16) TL_ML_LAUNCH(TT, 16);                 \
-  else if (D <= 32) TL_ML_LAUNCH(TT, 32);            \
-  else if (D <= 64) TL_ML_LAUNCH(TT, 64);            \
-  else if (D <= 128) TL_ML_LAUNCH(TT, 128);          \
-  else TL_ML_LAUNCH(TT, 256);
+#define TL_ML_LAUNCH(TT, DM, TBB, NTM)                                       \
+  do {                                                                       \
+    const size_t smem = sizeof(float) * (2 * TBB * D + 3 * TBB + TBB * nw);  \
+    hipLaunchKernelGGL((mlstm_seq_kernel<TT, DM, TBB, NTM>), grid, block,    \
+                       smem, stream, (const TT*)proj, ld, q_off, k_off,      \
+                       v_off, g_off, (const float*)gates,                    \
+                       (const float*)norm_w, (float*)S, (float*)n,           \
+                       (float*)m, (const int*)cu, (const int*)slots,         \
+                       (const int*)pos0, (TT*)out, H, D, V, cap, qscale,     \
+                       eps);                                                 \
+  } while (0)
+// register budget: blocks of up to 256 threads may use the full file;
+// wider blocks (vdim > 255) take short rounds
+#define TL_ML_D(TT)                                                \
+  if (nt > 256) {                                                  \
+    if (D <= 64) TL_ML_LAUNCH(TT, 64, 4, 1024);                    \
+    else TL_ML_LAUNCH(TT, 256, 4, 1024);                           \
+  } else if (D <= 32) TL_ML_LAUNCH(TT, 32, 16, 256);               \
+  else if (D <= 64) TL_ML_LAUNCH(TT, 64, 16, 256);                 \
+  else if (D <= 128) TL_ML_LAUNCH(TT, 128, 8, 256);                \
+  else TL_ML_LAUNCH(TT, 256, 4, 256);
   if (is_f32) {
     TL_ML_D(float)
   } else {

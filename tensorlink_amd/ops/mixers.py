@@ -60,6 +60,23 @@ class RaggedMeta:
         self.table = table.to(**i32).contiguous()
         self.max_kv = max((p + x for p, x in zip(self.pos0_h, self.new_h)),
                           default=0)
+        self._tiles = None
+        self._device = device
+
+    def query_tiles(self, size: int = 64) -> torch.Tensor:
+        """[n, 4] int32 rows (sequence, first flat token, count <= size,
+        first position): the step's tokens cut into per-sequence tiles for
+        the tiled attention kernel."""
+        if self._tiles is None:
+            rows = []
+            for b in range(self.B):
+                for o in range(0, self.new_h[b], size):
+                    rows.append([b, self.cu_h[b] + o,
+                                 min(size, self.new_h[b] - o),
+                                 self.pos0_h[b] + o])
+            self._tiles = torch.tensor(rows, dtype=torch.int32).reshape(
+                -1, 4).to(self._device)
+        return self._tiles
 
     @property
     def last_rows(self) -> List[int]:
@@ -201,6 +218,14 @@ def diff_attention(q: torch.Tensor, q_off: int, kpool: torch.Tensor,
     [H, 2, D] at column ``q_off``; returns [T, H*V] =
     unit_rms(a1 - lam * a2) * (1 - diff) per head."""
     if q.is_cuda:
+        if q.dtype == torch.bfloat16 and meta.T > meta.B:
+            # a prompt portion is in the step: 64-query MFMA tiles
+            out = torch.empty(q.shape[0], H * vpool.shape[3], device=q.device,
+                              dtype=q.dtype)
+            if _ext().diff_attn_tiles(q, q_off, kpool, vpool,
+                                      meta.query_tiles(), meta.table, lam,
+                                      out, H, D, scale, diff, eps):
+                return out
         return _ext().diff_attn_rows(q, q_off, kpool, vpool, meta.tok_seq,
                                      meta.tok_pos, meta.table, lam, H, D,
                                      scale, diff, eps)
