@@ -28,9 +28,9 @@ void tl_kv_append(const void* proj, int ld, int k_off, int v_off, void* kpool,
 int tl_diff_attn_rows(const void* q, int ldq, int q_off, const void* kpool,
                       const void* vpool, const void* tok_seq,
                       const void* tok_pos, const void* table, int P,
-                      const void* lam, void* out, int T, int H, int G, int D,
-                      int V, float scale, float diff, float eps, int is_f32,
-                      hipStream_t stream);
+                      const void* lam, void* out, void* part, int ns, int T,
+                      int H, int G, int D, int V, float scale, float diff,
+                      float eps, int is_f32, hipStream_t stream);
 int tl_diff_attn_tiles(const void* q, int ldq, int q_off, const void* kpool,
                        const void* vpool, const void* tiles, int n_tiles,
                        const void* table, int P, const void* lam, void* out,
@@ -194,10 +194,12 @@ void kv_append(Tensor proj, int64_t k_off, int64_t v_off, Tensor kpool,
                (int)T, G, DK, V, io_is_f32(proj), mix_stream());
 }
 
+// n_split > 1 spreads every row's keys over that many blocks (few rows
+// over long contexts: decoding) and merges them in a second kernel.
 Tensor diff_attn_rows(Tensor q, int64_t q_off, Tensor kpool, Tensor vpool,
                       Tensor tok_seq, Tensor tok_pos, Tensor table,
                       Tensor lam, int64_t H, int64_t D, double scale,
-                      double diff, double eps) {
+                      double diff, double eps, int64_t n_split) {
   MIX_IN(q);
   MIX_IN(kpool);
   MIX_IN(vpool);
@@ -219,11 +221,17 @@ Tensor diff_attn_rows(Tensor q, int64_t q_off, Tensor kpool, Tensor vpool,
               "ragged metadata");
   auto out = torch::empty({T, H * V}, q.options());
   if (T == 0) return out;
+  TORCH_CHECK(n_split >= 1 && n_split <= 64, "n_split out of range");
+  Tensor part;
+  if (n_split > 1)
+    part = torch::empty({T * H * n_split * (4 + 2 * V)},
+                        q.options().dtype(torch::kFloat));
   const int rc = tl_diff_attn_rows(
       q.data_ptr(), (int)ld, (int)q_off, kpool.data_ptr(), vpool.data_ptr(),
       tok_seq.data_ptr(), tok_pos.data_ptr(), table.data_ptr(),
-      (int)table.size(1), lam.data_ptr(), out.data_ptr(), (int)T, (int)H, G,
-      (int)D, V, (float)scale, (float)diff, (float)eps, io_is_f32(q),
+      (int)table.size(1), lam.data_ptr(), out.data_ptr(),
+      n_split > 1 ? part.data_ptr() : nullptr, (int)n_split, (int)T, (int)H,
+      G, (int)D, V, (float)scale, (float)diff, (float)eps, io_is_f32(q),
       mix_stream());
   TORCH_CHECK(rc == 0, "diff_attn_rows: shape outside the kernel's range "
                        "(vdim <= 512, heads divisible by kv heads)");

@@ -59,10 +59,11 @@ __global__ __launch_bounds__(BLOCK) void diff_attn_row_kernel(
     const T* __restrict__ kpool, const T* __restrict__ vpool,
     const int* __restrict__ tok_seq, const int* __restrict__ tok_pos,
     const int* __restrict__ table, int P, const float* __restrict__ lam_p,
-    T* __restrict__ out, int H, int G, int D, int V, float scale,
-    float diff, float eps) {
+    T* __restrict__ out, float* __restrict__ part, int H, int G, int D,
+    int V, float scale, float diff, float eps) {
   extern __shared__ float lds[];
   const int t = blockIdx.x, h = blockIdx.y;
+  const int ns = gridDim.z, z = blockIdx.z;   // key splits (flash-decode)
   const int g = h / (H / G);
   const int lane = threadIdx.x & (WAVE_SIZE - 1);
   const int wave = threadIdx.x / WAVE_SIZE;
@@ -84,7 +85,9 @@ __global__ __launch_bounds__(BLOCK) void diff_attn_row_kernel(
 #pragma unroll
   for (int r = 0; r < VR; ++r) a1[r] = a2[r] = 0.f;
 
-  for (int j0 = wave * WAVE_SIZE; j0 <= pos; j0 += NWAVE * WAVE_SIZE) {
+  const bool vec8 = (D % 8) == 0 && sizeof(T) == 2;
+  for (int j0 = (z * NWAVE + wave) * WAVE_SIZE; j0 <= pos;
+       j0 += ns * NWAVE * WAVE_SIZE) {
     const int j = j0 + lane;
     const bool valid = j <= pos;
     float s1 = -INFINITY, s2 = -INFINITY;
@@ -92,9 +95,22 @@ __global__ __launch_bounds__(BLOCK) void diff_attn_row_kernel(
       const int page = tab[j / PAGE];
       const T* kr = kpool + (((int64_t)page * G + g) * PAGE + (j % PAGE)) * DK;
       float x1 = 0.f, x2 = 0.f;
-      for (int d = 0; d < D; ++d) {
-        x1 += qs[d] * ldv<T>(kr + d);
-        x2 += qs[D + d] * ldv<T>(kr + D + d);
+      if (vec8) {
+        // 16-byte loads of 8 bf16 (rows are 16-byte aligned when D % 8 == 0)
+        const bf16x8* k8 = reinterpret_cast<const bf16x8*>(kr);
+        for (int d8 = 0; d8 < D / 8; ++d8) {
+          const bf16x8 a = k8[d8], b = k8[D / 8 + d8];
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            x1 += qs[d8 * 8 + e] * bf2f(a.v[e]);
+            x2 += qs[D + d8 * 8 + e] * bf2f(b.v[e]);
+          }
+        }
+      } else {
+        for (int d = 0; d < D; ++d) {
+          x1 += qs[d] * ldv<T>(kr + d);
+          x2 += qs[D + d] * ldv<T>(kr + D + d);
+        }
       }
       s1 = x1;
       s2 = x2;
@@ -159,6 +175,27 @@ __global__ __launch_bounds__(BLOCK) void diff_attn_row_kernel(
     L1 += f1[w] * stat[w * 4 + 1];
     L2 += f2[w] * stat[w * 4 + 3];
   }
+  if (ns > 1) {
+    // partial of this key split: (M1, L1, M2, L2 | A1[V] | A2[V]); the
+    // merge kernel finishes the row
+    float* pr = part + (((int64_t)t * H + h) * ns + z) * (4 + 2 * V);
+    if (threadIdx.x == 0) {
+      pr[0] = M1;
+      pr[1] = L1;
+      pr[2] = M2;
+      pr[3] = L2;
+    }
+    for (int c = threadIdx.x; c < V; c += BLOCK) {
+      float A1 = 0.f, A2 = 0.f;
+      for (int w = 0; w < NWAVE; ++w) {
+        A1 += f1[w] * accs[(w * 2 + 0) * V + c];
+        A2 += f2[w] * accs[(w * 2 + 1) * V + c];
+      }
+      pr[4 + c] = A1;
+      pr[4 + V + c] = A2;
+    }
+    return;
+  }
   const float lam = lam_p[0];
   // at most VR*64/BLOCK columns per thread; VR <= 8 -> 2
   float o[2];
@@ -190,6 +227,63 @@ __global__ __launch_bounds__(BLOCK) void diff_attn_row_kernel(
   }
 }
 
+// Merge the key splits of one (token, head): rescale every split's sums to
+// the common maximum, then lambda, unit RMS and (1 - diff) as in the row
+// kernel. One block of 256 threads per row; V <= 512.
+template <typename T>
+__global__ __launch_bounds__(BLOCK) void diff_attn_merge_kernel(
+    const float* __restrict__ part, const float* __restrict__ lam_p,
+    T* __restrict__ out, int ns, int V, float diff, float eps) {
+  __shared__ float red[NWAVE];
+  const int64_t row = blockIdx.x;
+  const float* pr = part + row * ns * (4 + 2 * V);
+  const int lane = threadIdx.x & (WAVE_SIZE - 1);
+  const int wave = threadIdx.x / WAVE_SIZE;
+  float M1 = -INFINITY, M2 = -INFINITY;
+  for (int z = 0; z < ns; ++z) {
+    M1 = fmaxf(M1, pr[z * (4 + 2 * V) + 0]);
+    M2 = fmaxf(M2, pr[z * (4 + 2 * V) + 2]);
+  }
+  float L1 = 0.f, L2 = 0.f;
+  float o[2] = {0.f, 0.f}, a1[2] = {0.f, 0.f}, a2[2] = {0.f, 0.f};
+  for (int z = 0; z < ns; ++z) {
+    const float* pz = pr + z * (4 + 2 * V);
+    const float f1 = pz[0] == -INFINITY ? 0.f : expf(pz[0] - M1);
+    const float f2 = pz[2] == -INFINITY ? 0.f : expf(pz[2] - M2);
+    L1 += f1 * pz[1];
+    L2 += f2 * pz[3];
+#pragma unroll
+    for (int r = 0; r < 2; ++r) {
+      const int c = threadIdx.x + r * BLOCK;
+      if (c < V) {
+        a1[r] += f1 * pz[4 + c];
+        a2[r] += f2 * pz[4 + V + c];
+      }
+    }
+  }
+  const float lam = lam_p[0];
+  float ss = 0.f;
+#pragma unroll
+  for (int r = 0; r < 2; ++r) {
+    const int c = threadIdx.x + r * BLOCK;
+    if (c < V) {
+      o[r] = a1[r] / L1 - lam * (a2[r] / L2);
+      ss += o[r] * o[r];
+    }
+  }
+  ss = wave_reduce_sum(ss);
+  if (lane == 0) red[wave] = ss;
+  __syncthreads();
+  float tot = 0.f;
+  for (int w = 0; w < NWAVE; ++w) tot += red[w];
+  const float rn = rsqrtf(tot / (float)V + eps) * (1.f - diff);
+#pragma unroll
+  for (int r = 0; r < 2; ++r) {
+    const int c = threadIdx.x + r * BLOCK;
+    if (c < V) stv<T>(out + row * V + c, o[r] * rn);
+  }
+}
+
 }  // namespace
 
 extern "C" {
@@ -216,22 +310,23 @@ void tl_kv_append(const void* proj, int ld, int k_off, int v_off, void* kpool,
 int tl_diff_attn_rows(const void* q, int ldq, int q_off, const void* kpool,
                       const void* vpool, const void* tok_seq,
                       const void* tok_pos, const void* table, int P,
-                      const void* lam, void* out, int T, int H, int G, int D,
-                      int V, float scale, float diff, float eps, int is_f32,
-                      hipStream_t stream) {
-  if (V > 512 || T <= 0 || H % G != 0) return 1;
+                      const void* lam, void* out, void* part, int ns, int T,
+                      int H, int G, int D, int V, float scale, float diff,
+                      float eps, int is_f32, hipStream_t stream) {
+  if (V > 512 || T <= 0 || H % G != 0 || ns < 1 || (ns > 1 && !part))
+    return 1;
   const size_t smem =
       sizeof(float) * (2 * D + NWAVE * 4 + NWAVE * 2 * V + NWAVE);
   if (smem > 64 * 1024) return 1;
-  dim3 grid(T, H), block(BLOCK);
+  dim3 grid(T, H, ns), block(BLOCK);
   const int vr = (V + WAVE_SIZE - 1) / WAVE_SIZE;
 #define TL_DA_LAUNCH(TT, VRR)                                                \
   hipLaunchKernelGGL((diff_attn_row_kernel<TT, VRR>), grid, block, smem,     \
                      stream, (const TT*)q, ldq, q_off, (const TT*)kpool,     \
                      (const TT*)vpool, (const int*)tok_seq,                  \
                      (const int*)tok_pos, (const int*)table, P,              \
-                     (const float*)lam, (TT*)out, H, G, D, V, scale, diff,   \
-                     eps)
+                     (const float*)lam, (TT*)out, (float*)part, H, G, D, V,  \
+                     scale, diff, eps)
 #define TL_DA_V(TT)                          \
   if (vr <= 1) TL_DA_LAUNCH(TT, 1);          \
   else if (vr <= 2) TL_DA_LAUNCH(TT, 2);     \
@@ -244,6 +339,17 @@ int tl_diff_attn_rows(const void* q, int ldq, int q_off, const void* kpool,
   }
 #undef TL_DA_V
 #undef TL_DA_LAUNCH
+  if (ns > 1) {
+    dim3 mgrid(T * H);
+    if (is_f32)
+      hipLaunchKernelGGL(diff_attn_merge_kernel<float>, mgrid, block, 0,
+                         stream, (const float*)part, (const float*)lam,
+                         (float*)out, ns, V, diff, eps);
+    else
+      hipLaunchKernelGGL(diff_attn_merge_kernel<bf16>, mgrid, block, 0,
+                         stream, (const float*)part, (const float*)lam,
+                         (bf16*)out, ns, V, diff, eps);
+  }
   return 0;
 }
 

@@ -50,16 +50,18 @@ __global__ __launch_bounds__(NTMAX) void mlstm_seq_kernel(
     const int* __restrict__ cu, const int* __restrict__ slots,
     const int* __restrict__ pos0, T* __restrict__ out, int H, int D, int V,
     float cap, float qscale, float eps) {
-  extern __shared__ float lds[];
+  extern __shared__ __align__(16) float lds[];
   const int h = blockIdx.x, b = blockIdx.y;
   const int c = threadIdx.x;
   const int nt = blockDim.x;
   const int nw = nt / WAVE_SIZE;
   const int lane = c & (WAVE_SIZE - 1), wave = c / WAVE_SIZE;
-  // lds: q[TB][D] | k[TB][D] | li[TB] | lf[TB] | nq[TB] | red[TB][nw]
+  // lds: q[TB][DMAX] | k[TB][DMAX] | li[TB] | lf[TB] | nq[TB] | red[TB][nw]
+  // (rows padded with zeros to DMAX: the inner loop carries no d < D test
+  // and reads float4; state entries beyond D stay zero)
   float* lq = lds;
-  float* lk = lq + TB * D;
-  float* lli = lk + TB * D;
+  float* lk = lq + TB * DMAX;
+  float* lli = lk + TB * DMAX;
   float* llf = lli + TB;
   float* lnq = llf + TB;
   float* red = lnq + TB;
@@ -88,11 +90,12 @@ __global__ __launch_bounds__(NTMAX) void mlstm_seq_kernel(
   for (int tb0 = t0; tb0 < t1; tb0 += TB) {
     const int cnt = min(TB, t1 - tb0);
     // ---- stage the round
-    for (int i = c; i < cnt * D; i += nt) {
-      const int tt = i / D, d = i - tt * D;
+    for (int i = c; i < cnt * DMAX; i += nt) {
+      const int tt = i / DMAX, d = i - tt * DMAX;
       const T* row = proj + (int64_t)(tb0 + tt) * ld;
-      lq[tt * D + d] = ldv<T>(row + q_off + h * D + d) * qscale;
-      lk[tt * D + d] = ldv<T>(row + k_off + h * D + d);
+      const bool in = d < D;
+      lq[i] = in ? ldv<T>(row + q_off + h * D + d) * qscale : 0.f;
+      lk[i] = in ? ldv<T>(row + k_off + h * D + d) : 0.f;
     }
     if (c < cnt) {
       const float gi = gates[(int64_t)(tb0 + c) * 2 * H + h];
@@ -124,15 +127,18 @@ __global__ __launch_bounds__(NTMAX) void mlstm_seq_kernel(
         const float bv = expf(li - m_new) * vreg[tt];
         m = m_new;
         em[tt] = expf(-m_new);
-        const float* qq = lq + tt * D;
-        const float* kk = lk + tt * D;
+        const float4* qq = reinterpret_cast<const float4*>(lq + tt * DMAX);
+        const float4* kk = reinterpret_cast<const float4*>(lk + tt * DMAX);
         float acc = 0.f;
 #pragma unroll
-        for (int d = 0; d < DMAX; ++d) {
-          if (d < D) {
-            s[d] = a * s[d] + bv * kk[d];
-            acc += s[d] * qq[d];
-          }
+        for (int d4 = 0; d4 < DMAX / 4; ++d4) {
+          const float4 k4 = kk[d4], q4 = qq[d4];
+          s[d4 * 4 + 0] = a * s[d4 * 4 + 0] + bv * k4.x;
+          s[d4 * 4 + 1] = a * s[d4 * 4 + 1] + bv * k4.y;
+          s[d4 * 4 + 2] = a * s[d4 * 4 + 2] + bv * k4.z;
+          s[d4 * 4 + 3] = a * s[d4 * 4 + 3] + bv * k4.w;
+          acc += s[d4 * 4 + 0] * q4.x + s[d4 * 4 + 1] * q4.y +
+                 s[d4 * 4 + 2] * q4.z + s[d4 * 4 + 3] * q4.w;
         }
         num[tt] = acc;
       }
@@ -189,7 +195,7 @@ int tl_mlstm_seq(const void* proj, int ld, int q_off, int k_off, int v_off,
   dim3 grid(H, B), block(nt);
 #define TL_ML_LAUNCH(TT, DM, TBB, NTM)                                       \
   do {                                                                       \
-    const size_t smem = sizeof(float) * (2 * TBB * D + 3 * TBB + TBB * nw);  \
+    const size_t smem = sizeof(float) * (2 * TBB * DM + 3 * TBB + TBB * nw);  \
     hipLaunchKernelGGL((mlstm_seq_kernel<TT, DM, TBB, NTM>), grid, block,    \
                        smem, stream, (const TT*)proj, ld, q_off, k_off,      \
                        v_off, g_off, (const float*)gates,                    \

@@ -17,6 +17,7 @@ share one forward pass.
 
 from __future__ import annotations
 
+import os
 from typing import List, Optional, Sequence
 
 import torch
@@ -218,7 +219,8 @@ def diff_attention(q: torch.Tensor, q_off: int, kpool: torch.Tensor,
     [H, 2, D] at column ``q_off``; returns [T, H*V] =
     unit_rms(a1 - lam * a2) * (1 - diff) per head."""
     if q.is_cuda:
-        if q.dtype == torch.bfloat16 and meta.T > meta.B:
+        if (q.dtype == torch.bfloat16 and meta.T > meta.B
+                and not os.environ.get("TL_NO_ATTN_TILES")):
             # a prompt portion is in the step: 64-query MFMA tiles
             out = torch.empty(q.shape[0], H * vpool.shape[3], device=q.device,
                               dtype=q.dtype)
@@ -226,9 +228,16 @@ def diff_attention(q: torch.Tensor, q_off: int, kpool: torch.Tensor,
                                       meta.query_tiles(), meta.table, lam,
                                       out, H, D, scale, diff, eps):
                 return out
+        # few rows over long contexts (decoding): spread each row's keys
+        # over several blocks so the chip is filled; a function of the
+        # step's shape only
+        n_split = 1
+        while (n_split < 16 and meta.T * H * n_split < 512
+               and meta.max_kv > 512 * n_split):
+            n_split *= 2
         return _ext().diff_attn_rows(q, q_off, kpool, vpool, meta.tok_seq,
                                      meta.tok_pos, meta.table, lam, H, D,
-                                     scale, diff, eps)
+                                     scale, diff, eps, n_split)
     G, V = kpool.shape[1], vpool.shape[3]
     T = q.shape[0]
     out = torch.empty(T, H, V)
