@@ -13,9 +13,10 @@
 //
 // One block serves one (sequence, head) and walks the sequence's tokens in
 // order, so the same kernel is the decode step (one token) and the exact
-// sequential prefill. Thread c < V owns column c of S in registers; thread
-// c == V owns n (the column a constant value 1 would produce), so n . q
-// falls out of the same dot product. A sequence whose cached length is zero
+// sequential prefill. Column thread c < V owns column c of S in registers
+// (split over DG thread groups along D); column thread c == V owns n (the
+// column a constant value 1 would produce), so n . q falls out of the same
+// dot product. A sequence whose cached length is zero
 // starts from the zero state without reading its slot: a reused slot needs
 // no clearing.
 
@@ -37,9 +38,12 @@ DEVINLINE float log_sigmoid(float x) {
 // TB tokens are staged per round: their q/k rows and capped gates go to
 // LDS in one sweep (one global-memory latency per round instead of one per
 // token), v and the output gate wait in registers, and the per-token
-// normaliser / RMS reductions of the whole round share one barrier.
-template <typename T, int DMAX, int TB, int NTMAX>
-__global__ __launch_bounds__(NTMAX) void mlstm_seq_kernel(
+// normaliser / RMS reductions of the whole round share the barriers.
+// DG thread groups split the D rows of every column (DMAX/DG state
+// registers per thread, DG times the waves to hide latency); their partial
+// read-outs meet in LDS once per round.
+template <typename T, int DMAX, int TB, int DG>
+__global__ __launch_bounds__(1024) void mlstm_seq_kernel(
     const T* __restrict__ proj, int ld, int q_off, int k_off, int v_off,
     int g_off,
     const float* __restrict__ gates,   // [Ttot, 2H] raw (input | forget)
@@ -50,13 +54,16 @@ __global__ __launch_bounds__(NTMAX) void mlstm_seq_kernel(
     const int* __restrict__ cu, const int* __restrict__ slots,
     const int* __restrict__ pos0, T* __restrict__ out, int H, int D, int V,
     float cap, float qscale, float eps) {
+  constexpr int DPER = DMAX / DG;
   extern __shared__ __align__(16) float lds[];
   const int h = blockIdx.x, b = blockIdx.y;
-  const int c = threadIdx.x;
   const int nt = blockDim.x;
-  const int nw = nt / WAVE_SIZE;
+  const int nc = nt / DG;                 // column threads per group
+  const int c = threadIdx.x % nc, dg = threadIdx.x / nc;
+  const int nw = nc / WAVE_SIZE;
   const int lane = c & (WAVE_SIZE - 1), wave = c / WAVE_SIZE;
-  // lds: q[TB][DMAX] | k[TB][DMAX] | li[TB] | lf[TB] | nq[TB] | red[TB][nw]
+  // lds: q[TB][DMAX] | k[TB][DMAX] | li[TB] | lf[TB] | nq[TB] | a[TB] |
+  //      b[TB] | em[TB] | m_end | red[TB][nw] | pnum[TB][DG][nc]
   // (rows padded with zeros to DMAX: the inner loop carries no d < D test
   // and reads float4; state entries beyond D stay zero)
   float* lq = lds;
@@ -64,25 +71,31 @@ __global__ __launch_bounds__(NTMAX) void mlstm_seq_kernel(
   float* lli = lk + TB * DMAX;
   float* llf = lli + TB;
   float* lnq = llf + TB;
-  float* red = lnq + TB;
+  float* la = lnq + TB;      // per token: exp(lf + m_prev - m), exp(li - m),
+  float* lb = la + TB;       //            exp(-m); then the round's last m
+  float* lem = lb + TB;
+  float* lmend = lem + TB;
+  float* red = lmend + 1;
+  float* pnum = red + TB * nw;
 
   const int t0 = cu[b], t1 = cu[b + 1];
   if (t0 >= t1) return;
   const int slot = slots[b];
   const bool fresh = pos0[b] == 0;
   const bool is_col = c < V, is_n = c == V;
+  const int d0 = dg * DPER;
 
-  float s[DMAX];
+  float s[DPER];
   float* S_base = S_pool + ((int64_t)slot * H + h) * (int64_t)D * V;
   float* n_base = n_pool + ((int64_t)slot * H + h) * D;
 #pragma unroll
-  for (int d = 0; d < DMAX; ++d) {
+  for (int i = 0; i < DPER; ++i) {
     float v = 0.f;
-    if (!fresh && d < D) {
-      if (is_col) v = S_base[(int64_t)d * V + c];
-      else if (is_n) v = n_base[d];
+    if (!fresh && d0 + i < D) {
+      if (is_col) v = S_base[(int64_t)(d0 + i) * V + c];
+      else if (is_n) v = n_base[d0 + i];
     }
-    s[d] = v;
+    s[i] = v;
   }
   float m = fresh ? 0.f : m_pool[(int64_t)slot * H + h];
   const float nw_c = is_col ? norm_w[h * V + c] : 0.f;
@@ -90,18 +103,19 @@ __global__ __launch_bounds__(NTMAX) void mlstm_seq_kernel(
   for (int tb0 = t0; tb0 < t1; tb0 += TB) {
     const int cnt = min(TB, t1 - tb0);
     // ---- stage the round
-    for (int i = c; i < cnt * DMAX; i += nt) {
+    for (int i = threadIdx.x; i < cnt * DMAX; i += nt) {
       const int tt = i / DMAX, d = i - tt * DMAX;
       const T* row = proj + (int64_t)(tb0 + tt) * ld;
       const bool in = d < D;
       lq[i] = in ? ldv<T>(row + q_off + h * D + d) * qscale : 0.f;
       lk[i] = in ? ldv<T>(row + k_off + h * D + d) : 0.f;
     }
-    if (c < cnt) {
-      const float gi = gates[(int64_t)(tb0 + c) * 2 * H + h];
-      const float gf = gates[(int64_t)(tb0 + c) * 2 * H + H + h];
-      lli[c] = cap * tanhf(gi / cap);
-      llf[c] = log_sigmoid(cap * tanhf(gf / cap));
+    if (threadIdx.x < cnt) {
+      const int tt = threadIdx.x;
+      const float gi = gates[(int64_t)(tb0 + tt) * 2 * H + h];
+      const float gf = gates[(int64_t)(tb0 + tt) * 2 * H + H + h];
+      lli[tt] = cap * tanhf(gi / cap);
+      llf[tt] = log_sigmoid(cap * tanhf(gf / cap));
     }
     float vreg[TB], greg[TB], num[TB], em[TB];
 #pragma unroll
@@ -111,47 +125,82 @@ __global__ __launch_bounds__(NTMAX) void mlstm_seq_kernel(
       if (tt < cnt && is_col) {
         const T* row = proj + (int64_t)(tb0 + tt) * ld;
         vreg[tt] = ldv<T>(row + v_off + h * V + c);
-        greg[tt] = ldv<T>(row + g_off + h * V + c);
+        if (dg == 0) greg[tt] = ldv<T>(row + g_off + h * V + c);
       }
     }
     __syncthreads();
+    // ---- the round's scale recurrence, once, by one thread per token
+    // (thread tt replays m over tokens 0..tt: at most TB cheap steps)
+    // instead of three exponentials per token in EVERY thread
+    if (threadIdx.x < cnt) {
+      const int tt = threadIdx.x;
+      float mp = m, mc = m;          // m before / after token tt
+      for (int j = 0; j <= tt; ++j) {
+        mp = mc;
+        mc = fmaxf(llf[j] + mc, lli[j]);
+      }
+      la[tt] = expf(llf[tt] + mp - mc);
+      lb[tt] = expf(lli[tt] - mc);
+      lem[tt] = expf(-mc);
+      if (tt == cnt - 1) lmend[0] = mc;
+    }
+    __syncthreads();
+    m = lmend[0];
     // ---- the recurrence, token by token, no barrier inside
 #pragma unroll
     for (int tt = 0; tt < TB; ++tt) {
       num[tt] = 0.f;
       em[tt] = 0.f;
       if (tt < cnt) {
-        const float li = lli[tt], lf = llf[tt];
-        const float m_new = fmaxf(lf + m, li);
-        const float a = expf(lf + m - m_new);
-        const float bv = expf(li - m_new) * vreg[tt];
-        m = m_new;
-        em[tt] = expf(-m_new);
-        const float4* qq = reinterpret_cast<const float4*>(lq + tt * DMAX);
-        const float4* kk = reinterpret_cast<const float4*>(lk + tt * DMAX);
-        float acc = 0.f;
+        const float a = la[tt];
+        const float bv = lb[tt] * vreg[tt];
+        em[tt] = lem[tt];
+        const float4* qq =
+            reinterpret_cast<const float4*>(lq + tt * DMAX + d0);
+        const float4* kk =
+            reinterpret_cast<const float4*>(lk + tt * DMAX + d0);
+        float ac0 = 0.f, ac1 = 0.f, ac2 = 0.f, ac3 = 0.f;
 #pragma unroll
-        for (int d4 = 0; d4 < DMAX / 4; ++d4) {
+        for (int d4 = 0; d4 < DPER / 4; ++d4) {
           const float4 k4 = kk[d4], q4 = qq[d4];
           s[d4 * 4 + 0] = a * s[d4 * 4 + 0] + bv * k4.x;
           s[d4 * 4 + 1] = a * s[d4 * 4 + 1] + bv * k4.y;
           s[d4 * 4 + 2] = a * s[d4 * 4 + 2] + bv * k4.z;
           s[d4 * 4 + 3] = a * s[d4 * 4 + 3] + bv * k4.w;
-          acc += s[d4 * 4 + 0] * q4.x + s[d4 * 4 + 1] * q4.y +
-                 s[d4 * 4 + 2] * q4.z + s[d4 * 4 + 3] * q4.w;
+          ac0 += s[d4 * 4 + 0] * q4.x;
+          ac1 += s[d4 * 4 + 1] * q4.y;
+          ac2 += s[d4 * 4 + 2] * q4.z;
+          ac3 += s[d4 * 4 + 3] * q4.w;
         }
-        num[tt] = acc;
+        num[tt] = (ac0 + ac1) + (ac2 + ac3);
+      }
+    }
+    // ---- the groups' partial read-outs meet
+    if (DG > 1) {
+#pragma unroll
+      for (int tt = 0; tt < TB; ++tt) pnum[(tt * DG + dg) * nc + c] = num[tt];
+      __syncthreads();
+      if (dg == 0) {
+#pragma unroll
+        for (int tt = 0; tt < TB; ++tt) {
+          float a = 0.f;
+#pragma unroll
+          for (int gq = 0; gq < DG; ++gq) a += pnum[(tt * DG + gq) * nc + c];
+          num[tt] = a;
+        }
       }
     }
     // ---- reductions of the whole round behind one barrier
+    if (dg == 0) {
 #pragma unroll
-    for (int tt = 0; tt < TB; ++tt) {
-      const float sq = wave_reduce_sum(is_col ? num[tt] * num[tt] : 0.f);
-      if (lane == 0) red[tt * nw + wave] = sq;
-      if (is_n) lnq[tt] = num[tt];
+      for (int tt = 0; tt < TB; ++tt) {
+        const float sq = wave_reduce_sum(is_col ? num[tt] * num[tt] : 0.f);
+        if (lane == 0) red[tt * nw + wave] = sq;
+        if (is_n) lnq[tt] = num[tt];
+      }
     }
     __syncthreads();
-    if (is_col) {
+    if (dg == 0 && is_col) {
 #pragma unroll
       for (int tt = 0; tt < TB; ++tt) {
         if (tt < cnt) {
@@ -166,16 +215,16 @@ __global__ __launch_bounds__(NTMAX) void mlstm_seq_kernel(
         }
       }
     }
-    __syncthreads();     // red / lq / lk are rewritten by the next round
+    __syncthreads();     // LDS is rewritten by the next round
   }
 #pragma unroll
-  for (int d = 0; d < DMAX; ++d) {
-    if (d < D) {
-      if (is_col) S_base[(int64_t)d * V + c] = s[d];
-      else if (is_n) n_base[d] = s[d];
+  for (int i = 0; i < DPER; ++i) {
+    if (d0 + i < D) {
+      if (is_col) S_base[(int64_t)(d0 + i) * V + c] = s[i];
+      else if (is_n) n_base[d0 + i] = s[i];
     }
   }
-  if (c == 0) m_pool[(int64_t)slot * H + h] = m;
+  if (threadIdx.x == 0) m_pool[(int64_t)slot * H + h] = m;
 }
 
 }  // namespace
@@ -190,30 +239,31 @@ int tl_mlstm_seq(const void* proj, int ld, int q_off, int k_off, int v_off,
                  float cap, float qscale, float eps, int is_f32,
                  hipStream_t stream) {
   if (D > 256 || V + 1 > 1024 || B < 1) return 1;
-  const int nt = ((V + 1 + WAVE_SIZE - 1) / WAVE_SIZE) * WAVE_SIZE;
-  const int nw = nt / WAVE_SIZE;
-  dim3 grid(H, B), block(nt);
-#define TL_ML_LAUNCH(TT, DM, TBB, NTM)                                       \
+  const int nc = ((V + 1 + WAVE_SIZE - 1) / WAVE_SIZE) * WAVE_SIZE;
+  const int nw = nc / WAVE_SIZE;
+  dim3 grid(H, B);
+#define TL_ML_LAUNCH(TT, DM, TBB, DGG)                                       \
   do {                                                                       \
-    const size_t smem = sizeof(float) * (2 * TBB * DM + 3 * TBB + TBB * nw);  \
-    hipLaunchKernelGGL((mlstm_seq_kernel<TT, DM, TBB, NTM>), grid, block,    \
-                       smem, stream, (const TT*)proj, ld, q_off, k_off,      \
-                       v_off, g_off, (const float*)gates,                    \
+    const size_t smem = sizeof(float) * (2 * TBB * DM + 6 * TBB + 4 + TBB * nw + \
+                                         (DGG > 1 ? TBB * DGG * nc : 0));    \
+    hipLaunchKernelGGL((mlstm_seq_kernel<TT, DM, TBB, DGG>), grid,           \
+                       dim3(nc * DGG), smem, stream, (const TT*)proj, ld,    \
+                       q_off, k_off, v_off, g_off, (const float*)gates,      \
                        (const float*)norm_w, (float*)S, (float*)n,           \
                        (float*)m, (const int*)cu, (const int*)slots,         \
                        (const int*)pos0, (TT*)out, H, D, V, cap, qscale,     \
                        eps);                                                 \
   } while (0)
-// register budget: blocks of up to 256 threads may use the full file;
-// wider blocks (vdim > 255) take short rounds
+// up to 256 column threads: four D-groups per column; wider heads keep one
+// group and short rounds
 #define TL_ML_D(TT)                                                \
-  if (nt > 256) {                                                  \
-    if (D <= 64) TL_ML_LAUNCH(TT, 64, 4, 1024);                    \
-    else TL_ML_LAUNCH(TT, 256, 4, 1024);                           \
-  } else if (D <= 32) TL_ML_LAUNCH(TT, 32, 16, 256);               \
-  else if (D <= 64) TL_ML_LAUNCH(TT, 64, 16, 256);                 \
-  else if (D <= 128) TL_ML_LAUNCH(TT, 128, 8, 256);                \
-  else TL_ML_LAUNCH(TT, 256, 4, 256);
+  if (nc > 256) {                                                  \
+    if (D <= 64) TL_ML_LAUNCH(TT, 64, 4, 1);                       \
+    else TL_ML_LAUNCH(TT, 256, 4, 1);                              \
+  } else if (D <= 32) TL_ML_LAUNCH(TT, 32, 8, 4);                  \
+  else if (D <= 64) TL_ML_LAUNCH(TT, 64, 8, 4);                    \
+  else if (D <= 128) TL_ML_LAUNCH(TT, 128, 8, 4);                  \
+  else TL_ML_LAUNCH(TT, 256, 8, 4);
   if (is_f32) {
     TL_ML_D(float)
   } else {

@@ -164,7 +164,17 @@ def main():
                          "(default: seeded random init)")
     ex.add_argument("--seed", type=int, default=0)
 
+    sub.add_parser("replay", help="replay a JSON-lines token trace "
+                   "through the batcher and write the requested logits "
+                   "(same flags as bin/trace_run)")
+
     args, extra = p.parse_known_args()
+    if args.cmd == "replay":
+        import runpy
+        here = os.path.dirname(os.path.abspath(__file__))
+        sys.argv = [os.path.join(here, "bin", "trace_run")] + extra
+        runpy.run_path(sys.argv[0], run_name="__main__")
+        return
     if args.cmd == "serve":
         cmd_serve(args)
     elif args.cmd == "plan":
