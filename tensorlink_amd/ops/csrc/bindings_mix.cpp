@@ -19,8 +19,13 @@ int tl_mlstm_seq(const void* proj, int ld, int q_off, int k_off, int v_off,
                  int g_off, const void* gates, const void* norm_w, void* S,
                  void* n, void* m, const void* cu, const void* slots,
                  const void* pos0, void* out, int B, int H, int D, int V,
-                 float cap, float qscale, float eps, int is_f32,
-                 hipStream_t stream);
+                 float cap, float qscale, float eps, void* F, int summary,
+                 int is_f32, hipStream_t stream);
+int tl_mlstm_chain(void* S_tmp, void* n_tmp, void* m_tmp, const void* F_tmp,
+                   void* S, void* n, void* m, const void* chunk_base,
+                   const void* n_chunks, const void* slots, const void* pos0,
+                   int B, int max_chunks, int H, int D, int V,
+                   hipStream_t stream);
 void tl_kv_append(const void* proj, int ld, int k_off, int v_off, void* kpool,
                   void* vpool, const void* tok_seq, const void* tok_pos,
                   const void* table, int P, int T, int G, int DK, int V,
@@ -131,7 +136,10 @@ Tensor mlstm_seq(Tensor proj, int64_t q_off, int64_t k_off, int64_t v_off,
                  int64_t g_off, Tensor gates, Tensor norm_w, Tensor S,
                  Tensor n, Tensor m, Tensor cu, Tensor slots, Tensor pos0,
                  int64_t H, int64_t D, int64_t V, double cap, double qscale,
-                 double eps) {
+                 double eps, c10::optional<Tensor> F_sum) {
+  // F_sum given = summary mode: every ragged entry is run from the empty
+  // state, no output is produced, its slot receives the entry's summary
+  // and F_sum [slots, H] the sum of its log forget gates
   MIX_IN(proj);
   MIX_F32(gates);
   MIX_F32(norm_w);
@@ -155,17 +163,58 @@ Tensor mlstm_seq(Tensor proj, int64_t q_off, int64_t k_off, int64_t v_off,
               "S pool must be [slots, H, D, V]");
   TORCH_CHECK(n.numel() == S.size(0) * H * D && m.numel() == S.size(0) * H,
               "n / m pools do not match S");
-  auto out = torch::empty({T, H * V}, proj.options());
+  const bool summary = F_sum.has_value();
+  if (summary) {
+    MIX_F32(F_sum.value());
+    TORCH_CHECK(F_sum->numel() == S.size(0) * H, "F_sum must be [slots, H]");
+  }
+  auto out = torch::empty({summary ? 0 : T, H * V}, proj.options());
   if (T == 0 || B == 0) return out;
   const int rc = tl_mlstm_seq(
       proj.data_ptr(), (int)ld, (int)q_off, (int)k_off, (int)v_off,
       (int)g_off, gates.data_ptr(), norm_w.data_ptr(), S.data_ptr(),
       n.data_ptr(), m.data_ptr(), cu.data_ptr(), slots.data_ptr(),
       pos0.data_ptr(), out.data_ptr(), B, (int)H, (int)D, (int)V, (float)cap,
-      (float)qscale, (float)eps, io_is_f32(proj), mix_stream());
+      (float)qscale, (float)eps, summary ? F_sum->data_ptr() : nullptr,
+      summary ? 1 : 0, io_is_f32(proj), mix_stream());
   TORCH_CHECK(rc == 0, "mlstm_seq: head sizes outside the kernel's range "
                        "(dim <= 256, vdim <= 1023)");
   return out;
+}
+
+void mlstm_chain(Tensor S_tmp, Tensor n_tmp, Tensor m_tmp, Tensor F_tmp,
+                 Tensor S, Tensor n, Tensor m, Tensor chunk_base,
+                 Tensor n_chunks, Tensor slots, Tensor pos0,
+                 int64_t max_chunks) {
+  MIX_F32(S_tmp);
+  MIX_F32(n_tmp);
+  MIX_F32(m_tmp);
+  MIX_F32(F_tmp);
+  MIX_F32(S);
+  MIX_F32(n);
+  MIX_F32(m);
+  MIX_I32(chunk_base);
+  MIX_I32(n_chunks);
+  MIX_I32(slots);
+  MIX_I32(pos0);
+  TORCH_CHECK(S.dim() == 4 && S_tmp.dim() == 4, "S pools must be 4-d");
+  const int H = S.size(1), D = S.size(2), V = S.size(3);
+  TORCH_CHECK(S_tmp.size(1) == H && S_tmp.size(2) == D && S_tmp.size(3) == V,
+              "chunk pool does not match the slot pool");
+  const int64_t NC = S_tmp.size(0);
+  TORCH_CHECK(n_tmp.numel() == NC * H * D && m_tmp.numel() == NC * H &&
+                  F_tmp.numel() == NC * H,
+              "chunk n / m / F pools do not match");
+  const int B = slots.size(0);
+  TORCH_CHECK(chunk_base.size(0) == B && n_chunks.size(0) == B &&
+                  pos0.size(0) == B,
+              "per-sequence chunk metadata");
+  const int rc = tl_mlstm_chain(
+      S_tmp.data_ptr(), n_tmp.data_ptr(), m_tmp.data_ptr(), F_tmp.data_ptr(),
+      S.data_ptr(), n.data_ptr(), m.data_ptr(), chunk_base.data_ptr(),
+      n_chunks.data_ptr(), slots.data_ptr(), pos0.data_ptr(), B,
+      (int)max_chunks, H, D, V, mix_stream());
+  TORCH_CHECK(rc == 0, "mlstm_chain: too many chunks in one sequence");
 }
 
 void kv_append(Tensor proj, int64_t k_off, int64_t v_off, Tensor kpool,
@@ -283,6 +332,8 @@ void register_mix_ops(pybind11::module& mod) {
   mod.def("relu_sq", &relu_sq, "relu(x)^2");
   mod.def("mlstm_seq", &mlstm_seq,
           "matrix-memory recurrence over ragged sequences (slot state)");
+  mod.def("mlstm_chain", &mlstm_chain,
+          "chain per-chunk mLSTM summaries into per-chunk start states");
   mod.def("kv_append", &kv_append, "scatter new K/V rows into page pools");
   mod.def("diff_attn_tiles", &diff_attn_tiles,
           "differential attention on MFMA, 64-query tiles, paged KV (bf16)");

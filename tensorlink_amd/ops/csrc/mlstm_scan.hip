@@ -53,7 +53,13 @@ __global__ __launch_bounds__(1024) void mlstm_seq_kernel(
     float* __restrict__ m_pool,        // [slots, H]
     const int* __restrict__ cu, const int* __restrict__ slots,
     const int* __restrict__ pos0, T* __restrict__ out, int H, int D, int V,
-    float cap, float qscale, float eps) {
+    float cap, float qscale, float eps,
+    float* __restrict__ F_pool,        // [slots, H] (summary mode) or null
+    int summary) {
+  // summary mode: the block runs its tokens from the EMPTY state with
+  // m = -inf, writes no output, and leaves in its slot the tokens' joint
+  // contribution (S, n scaled by exp(-m), m = their own maximum) plus the
+  // sum of their log forget gates in F_pool: one link of the chunk chain.
   constexpr int DPER = DMAX / DG;
   extern __shared__ __align__(16) float lds[];
   const int h = blockIdx.x, b = blockIdx.y;
@@ -74,16 +80,17 @@ __global__ __launch_bounds__(1024) void mlstm_seq_kernel(
   float* la = lnq + TB;      // per token: exp(lf + m_prev - m), exp(li - m),
   float* lb = la + TB;       //            exp(-m); then the round's last m
   float* lem = lb + TB;
-  float* lmend = lem + TB;
-  float* red = lmend + 1;
+  float* lmend = lem + TB;   // [0] round's last m, [1] running sum of lf
+  float* red = lmend + 2;
   float* pnum = red + TB * nw;
 
   const int t0 = cu[b], t1 = cu[b + 1];
   if (t0 >= t1) return;
   const int slot = slots[b];
-  const bool fresh = pos0[b] == 0;
+  const bool fresh = summary || pos0[b] == 0;
   const bool is_col = c < V, is_n = c == V;
   const int d0 = dg * DPER;
+  if (threadIdx.x == 0) lmend[1] = 0.f;
 
   float s[DPER];
   float* S_base = S_pool + ((int64_t)slot * H + h) * (int64_t)D * V;
@@ -97,7 +104,8 @@ __global__ __launch_bounds__(1024) void mlstm_seq_kernel(
     }
     s[i] = v;
   }
-  float m = fresh ? 0.f : m_pool[(int64_t)slot * H + h];
+  float m = summary ? -INFINITY
+                    : (fresh ? 0.f : m_pool[(int64_t)slot * H + h]);
   const float nw_c = is_col ? norm_w[h * V + c] : 0.f;
 
   for (int tb0 = t0; tb0 < t1; tb0 += TB) {
@@ -142,7 +150,12 @@ __global__ __launch_bounds__(1024) void mlstm_seq_kernel(
       la[tt] = expf(llf[tt] + mp - mc);
       lb[tt] = expf(lli[tt] - mc);
       lem[tt] = expf(-mc);
-      if (tt == cnt - 1) lmend[0] = mc;
+      if (tt == cnt - 1) {
+        lmend[0] = mc;
+        float f = lmend[1];
+        for (int j = 0; j < cnt; ++j) f += llf[j];
+        lmend[1] = f;
+      }
     }
     __syncthreads();
     m = lmend[0];
@@ -174,6 +187,10 @@ __global__ __launch_bounds__(1024) void mlstm_seq_kernel(
         }
         num[tt] = (ac0 + ac1) + (ac2 + ac3);
       }
+    }
+    if (summary) {           // block-uniform: no read-out, next round
+      __syncthreads();
+      continue;
     }
     // ---- the groups' partial read-outs meet
     if (DG > 1) {
@@ -224,7 +241,65 @@ __global__ __launch_bounds__(1024) void mlstm_seq_kernel(
       else if (is_n) n_base[d0 + i] = s[i];
     }
   }
-  if (threadIdx.x == 0) m_pool[(int64_t)slot * H + h] = m;
+  if (threadIdx.x == 0) {
+    m_pool[(int64_t)slot * H + h] = m;
+    if (summary) F_pool[(int64_t)slot * H + h] = lmend[1];
+  }
+}
+
+// Chain the chunk summaries of every sequence: walking a sequence's chunks
+// in order with the running state (S, n, m) — the slot's, or empty —
+//     m' = max(F_c + m, m_c)
+//     X' = exp(F_c + m - m') X + exp(m_c - m') dX_c          (X = S and n)
+// where (dX_c, m_c, F_c) is chunk c's summary. Each chunk's entry is
+// REPLACED by the state BEFORE the chunk (what the read-out pass of that
+// chunk starts from); the state after the last chunk goes to the slot.
+// The same m as token-by-token: max is associative. One block per
+// (head, sequence); threads own elements, chunks are walked sequentially.
+constexpr int CHAIN_MAX = 2048;
+
+__global__ __launch_bounds__(256) void mlstm_chain_kernel(
+    float* __restrict__ S_tmp, float* __restrict__ n_tmp,
+    float* __restrict__ m_tmp, const float* __restrict__ F_tmp,
+    float* __restrict__ S_pool, float* __restrict__ n_pool,
+    float* __restrict__ m_pool, const int* __restrict__ chunk_base,
+    const int* __restrict__ n_chunks, const int* __restrict__ slots,
+    const int* __restrict__ pos0, int H, int D, int V) {
+  __shared__ float ca[CHAIN_MAX], cb[CHAIN_MAX];
+  const int h = blockIdx.x, b = blockIdx.y;
+  const int c0 = chunk_base[b], C = n_chunks[b];
+  if (C <= 0) return;
+  const int slot = slots[b];
+  const bool fresh = pos0[b] == 0;
+  if (threadIdx.x == 0) {
+    float m = fresh ? 0.f : m_pool[(int64_t)slot * H + h];
+    for (int c = 0; c < C; ++c) {
+      const int64_t ci = (int64_t)(c0 + c) * H + h;
+      const float mc = m_tmp[ci], f = F_tmp[ci];
+      const float mn = fmaxf(f + m, mc);
+      ca[c] = expf(f + m - mn);
+      cb[c] = expf(mc - mn);
+      m_tmp[ci] = m;                 // scale before the chunk
+      m = mn;
+    }
+    m_pool[(int64_t)slot * H + h] = m;
+  }
+  __syncthreads();
+  const int DV = D * V;
+  for (int e = threadIdx.x; e < DV + D; e += blockDim.x) {
+    const bool isS = e < DV;
+    float* pool = isS ? S_pool + ((int64_t)slot * H + h) * DV + e
+                      : n_pool + ((int64_t)slot * H + h) * D + (e - DV);
+    float x = fresh ? 0.f : *pool;
+    for (int c = 0; c < C; ++c) {
+      const int64_t ci = (int64_t)(c0 + c) * H + h;
+      float* t = isS ? S_tmp + ci * DV + e : n_tmp + ci * D + (e - DV);
+      const float d = *t;
+      *t = x;
+      x = ca[c] * x + cb[c] * d;
+    }
+    *pool = x;
+  }
 }
 
 }  // namespace
@@ -236,15 +311,16 @@ int tl_mlstm_seq(const void* proj, int ld, int q_off, int k_off, int v_off,
                  int g_off, const void* gates, const void* norm_w, void* S,
                  void* n, void* m, const void* cu, const void* slots,
                  const void* pos0, void* out, int B, int H, int D, int V,
-                 float cap, float qscale, float eps, int is_f32,
-                 hipStream_t stream) {
+                 float cap, float qscale, float eps, void* F, int summary,
+                 int is_f32, hipStream_t stream) {
+  if (summary && !F) return 1;
   if (D > 256 || V + 1 > 1024 || B < 1) return 1;
   const int nc = ((V + 1 + WAVE_SIZE - 1) / WAVE_SIZE) * WAVE_SIZE;
   const int nw = nc / WAVE_SIZE;
   dim3 grid(H, B);
 #define TL_ML_LAUNCH(TT, DM, TBB, DGG)                                       \
   do {                                                                       \
-    const size_t smem = sizeof(float) * (2 * TBB * DM + 6 * TBB + 4 + TBB * nw + \
+    const size_t smem = sizeof(float) * (2 * TBB * DM + 6 * TBB + 8 + TBB * nw + \
                                          (DGG > 1 ? TBB * DGG * nc : 0));    \
     hipLaunchKernelGGL((mlstm_seq_kernel<TT, DM, TBB, DGG>), grid,           \
                        dim3(nc * DGG), smem, stream, (const TT*)proj, ld,    \
@@ -252,7 +328,7 @@ int tl_mlstm_seq(const void* proj, int ld, int q_off, int k_off, int v_off,
                        (const float*)norm_w, (float*)S, (float*)n,           \
                        (float*)m, (const int*)cu, (const int*)slots,         \
                        (const int*)pos0, (TT*)out, H, D, V, cap, qscale,     \
-                       eps);                                                 \
+                       eps, (float*)F, summary);                             \
   } while (0)
 // up to 256 column threads: four D-groups per column; wider heads keep one
 // group and short rounds
@@ -271,6 +347,22 @@ int tl_mlstm_seq(const void* proj, int ld, int q_off, int k_off, int v_off,
   }
 #undef TL_ML_D
 #undef TL_ML_LAUNCH
+  return 0;
+}
+
+// chunk_base/n_chunks/slots/pos0 are per sequence; returns 1 if a sequence
+// has more chunks than the kernel's table holds
+int tl_mlstm_chain(void* S_tmp, void* n_tmp, void* m_tmp, const void* F_tmp,
+                   void* S, void* n, void* m, const void* chunk_base,
+                   const void* n_chunks, const void* slots, const void* pos0,
+                   int B, int max_chunks, int H, int D, int V,
+                   hipStream_t stream) {
+  if (max_chunks > CHAIN_MAX || B < 1) return 1;
+  hipLaunchKernelGGL(mlstm_chain_kernel, dim3(H, B), dim3(256), 0, stream,
+                     (float*)S_tmp, (float*)n_tmp, (float*)m_tmp,
+                     (const float*)F_tmp, (float*)S, (float*)n, (float*)m,
+                     (const int*)chunk_base, (const int*)n_chunks,
+                     (const int*)slots, (const int*)pos0, H, D, V);
   return 0;
 }
 

@@ -23,6 +23,7 @@ from typing import List, Optional, Sequence
 import torch
 
 PAGE = 128
+SCAN_CHUNK = 64      # tokens per chunk of the chunk-parallel recurrence
 
 
 class RaggedMeta:
@@ -78,6 +79,32 @@ class RaggedMeta:
             self._tiles = torch.tensor(rows, dtype=torch.int32).reshape(
                 -1, 4).to(self._device)
         return self._tiles
+
+    def scan_chunks(self, size: int):
+        """The step's tokens cut into per-sequence chunks of ``size`` for
+        the chunk-parallel recurrence: (cu [NC+1], chunk ids [NC], ones
+        [NC], first chunk per sequence [B], chunk count per sequence [B],
+        NC, largest count) — index tensors on the device, built once per
+        step and shared by all layers."""
+        hit = self.__dict__.setdefault("_chunks", {}).get(size)
+        if hit is None:
+            cu, base, cnt = [0], [], []
+            for b in range(self.B):
+                base.append(len(cu) - 1)
+                n = 0
+                for o in range(0, self.new_h[b], size):
+                    cu.append(self.cu_h[b] + min(o + size, self.new_h[b]))
+                    n += 1
+                cnt.append(n)
+            nc = len(cu) - 1
+            packed = torch.tensor(cu + list(range(nc)) + [1] * nc + base
+                                  + cnt, dtype=torch.int32).to(self._device)
+            o1, o2, o3 = nc + 1, 2 * nc + 1, 3 * nc + 1
+            hit = (packed[:o1], packed[o1:o2], packed[o2:o3],
+                   packed[o3:o3 + self.B], packed[o3 + self.B:], nc,
+                   max(cnt, default=0))
+            self._chunks[size] = hit
+        return hit
 
     @property
     def last_rows(self) -> List[int]:
@@ -149,10 +176,36 @@ def mlstm_scan(proj: torch.Tensor, offs, gates: torch.Tensor,
     q_off, k_off, v_off, g_off = offs
     qscale = D ** -0.5
     if proj.is_cuda:
-        return _ext().mlstm_seq(proj, q_off, k_off, v_off, g_off,
-                                gates.contiguous(), norm_w, S, n, m,
-                                meta.cu, meta.slots, meta.pos0, H, D, V,
-                                cap, qscale, eps)
+        C = _ext()
+        gates = gates.contiguous()
+        chunk = SCAN_CHUNK
+        while max(meta.new_h) * H * D * V * 4 // chunk > (1 << 30):
+            chunk *= 2                   # bound the chunk-state scratch
+        if (max(meta.new_h) >= 4 * chunk
+                and not os.environ.get("TL_NO_SCAN_CHUNKS")):
+            # long prompt portions: chunk-parallel form. (1) every chunk's
+            # own summary from the empty state, all chunks in parallel;
+            # (2) a cheap sequential chain turns summaries into the state
+            # BEFORE each chunk and updates the slots; (3) every chunk's
+            # read-out from its start state, all chunks in parallel.
+            cu_c, ids_c, ones_c, base, cnt, nc, cmax = meta.scan_chunks(chunk)
+            if cmax <= 2048:
+                f32 = dict(device=proj.device, dtype=torch.float32)
+                S_t = torch.empty(nc, H, D, V, **f32)
+                n_t = torch.empty(nc, H, D, **f32)
+                m_t = torch.empty(nc, H, **f32)
+                F_t = torch.empty(nc, H, **f32)
+                C.mlstm_seq(proj, q_off, k_off, v_off, g_off, gates, norm_w,
+                            S_t, n_t, m_t, cu_c, ids_c, ones_c, H, D, V, cap,
+                            qscale, eps, F_t)
+                C.mlstm_chain(S_t, n_t, m_t, F_t, S, n, m, base, cnt,
+                              meta.slots, meta.pos0, cmax)
+                return C.mlstm_seq(proj, q_off, k_off, v_off, g_off, gates,
+                                   norm_w, S_t, n_t, m_t, cu_c, ids_c,
+                                   ones_c, H, D, V, cap, qscale, eps, None)
+        return C.mlstm_seq(proj, q_off, k_off, v_off, g_off, gates, norm_w,
+                           S, n, m, meta.cu, meta.slots, meta.pos0, H, D, V,
+                           cap, qscale, eps, None)
     T = proj.shape[0]
     pf = proj.float()
     q = pf[:, q_off:q_off + H * D].view(T, H, D) * qscale

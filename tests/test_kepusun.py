@@ -318,11 +318,14 @@ def _one_seq_meta(cache, n, pos0, device, slot=0):
     return mx.RaggedMeta([n], [pos0], [slot], cache.table[[slot]], device)
 
 
+@pytest.mark.parametrize("T", [37, 333])
 @pytest.mark.parametrize("device,dtype", ALL)
-def test_mlstm_mixer_against_oracle(device, dtype):
+def test_mlstm_mixer_against_oracle(device, dtype, T):
     """The mixer alone, whole sequence and token by token through the
     state slot; biases push some tokens onto each branch of the
-    normaliser max(|n.q|, exp(-m))."""
+    normaliser max(|n.q|, exp(-m)). The long sequence takes the
+    chunk-parallel form on the GPU (summaries, chain, read-out), also as a
+    continuation of a state left by an earlier portion."""
     from tensorlink_amd.models.mixers import MLSTMMixer
     g = torch.Generator().manual_seed(3)
     W, H, D, V, cap, eps = 48, 3, 20, 28, 6.0, 1e-5
@@ -334,7 +337,6 @@ def test_mlstm_mixer_against_oracle(device, dtype):
          "m.i": r(H, W, std=.5), "m.f": r(H, W, std=.5),
          "m.i.b": torch.tensor([-6.0, 0.0, 4.0]),
          "m.f.b": torch.tensor([3.0, -1.0, 0.5])}
-    T = 37
     h = r(T, W)
     mc = {"heads": H, "dim": D, "vdim": V, "gate_cap": cap}
     want = O.mlstm_sequence(h, P, "m.", mc, eps)
@@ -347,17 +349,26 @@ def test_mlstm_mixer_against_oracle(device, dtype):
         mod.norm.copy_(P["m.norm"])
         mod.o_proj.weight.copy_(P["m.o"])
     mod.to(device=device, dtype=dtype)
-    cache = HybridSlotCache([mod.cache_spec()], 3, 4, 256, device, dtype)
+    cache = HybridSlotCache([mod.cache_spec()], 4, 12, 512, device, dtype)
     hd = h.to(device=device, dtype=dtype)
+    cut = 11 if T < 100 else 40         # second portion of 293 tokens
     with torch.no_grad():
         whole = mod(hd, _one_seq_meta(cache, T, 0, device, slot=1), cache, 0)
         steps = [mod(hd[t:t + 1], _one_seq_meta(cache, 1, t, device, slot=2),
                      cache, 0) for t in range(T)]
+        parts = [mod(hd[:cut], _one_seq_meta(cache, cut, 0, device, slot=3),
+                     cache, 0),
+                 mod(hd[cut:], _one_seq_meta(cache, T - cut, cut, device,
+                                             slot=3), cache, 0)]
     scale = float(want.abs().max())
     t_ = 2e-5 if dtype == torch.float32 else 3e-2
-    assert float((whole.float().cpu() - want).abs().max()) < t_ * scale
-    assert float((torch.cat(steps).float().cpu() - want).abs().max()) \
-        < t_ * scale
+    for got in (whole, torch.cat(steps), torch.cat(parts)):
+        assert float((got.float().cpu() - want).abs().max()) < t_ * scale
+    # the slot state after the whole / cut / stepped runs agrees
+    for a, b_ in zip(cache.state[0], cache.state[0]):
+        for s2 in (2, 3):
+            assert torch.allclose(a[1].cpu(), b_[s2].cpu(), rtol=1e-3,
+                                  atol=1e-4 * float(a[1].abs().max()))
 
 
 @pytest.mark.parametrize("dims", [(4, 2, 8, 12), (4, 2, 16, 32),
@@ -503,6 +514,23 @@ def test_mixed_batch_and_reuse_of_slots_and_pages(tmp_path_factory, device,
     for r in toks:
         assert at[r] == lens[r]
         assert close(torch.cat(got[r]), want[r], dtype), r
+
+
+@pytest.mark.parametrize("device,dtype", ALL)
+def test_long_prompts_in_one_batch(tmp_path_factory, device, dtype):
+    """Prompts long enough for the chunk-parallel recurrence and several
+    attention tiles, two of unequal length in one step, the longer one
+    continued by a second long portion."""
+    runner, P, cfg = model(tmp_path_factory, cfg_tiles, device, dtype)
+    ta, tb = tokens(cfg, 610, 31), tokens(cfg, 77, 32)
+    wa = reference(runner, ta, P, cfg, dtype)
+    wb = reference(runner, tb, P, cfg, dtype)
+    b = batcher(runner, max_ctx=1024)
+    o1 = b.forced_step([("a", ta[:300], list(range(300))),
+                        ("b", tb, list(range(77)))], ["b"])
+    o2 = b.forced_step([("a", ta[300:], list(range(310)))], ["a"])
+    assert close(torch.cat([o1[:300], o2]), wa, dtype)
+    assert close(o1[300:], wb, dtype)
 
 
 @pytest.mark.parametrize("device,dtype", [CPU32, GPU32])
