@@ -22,6 +22,7 @@
 namespace {
 
 constexpr int PAGE = 128;
+static_assert(PAGE % WAVE_SIZE == 0, "a key tile must not straddle pages");
 constexpr int NWAVE = 4;
 constexpr int BLOCK = NWAVE * WAVE_SIZE;
 
@@ -91,9 +92,13 @@ __global__ __launch_bounds__(BLOCK) void diff_attn_row_kernel(
     const int j = j0 + lane;
     const bool valid = j <= pos;
     float s1 = -INFINITY, s2 = -INFINITY;
+    // a 64-key tile starts at a multiple of 64 and so lies inside ONE
+    // 128-position page: one table lookup per tile, and the value loads
+    // below do not wait on per-key lookups
+    const int64_t tile_row =
+        ((int64_t)tab[j0 / PAGE] * G + g) * PAGE + (j0 % PAGE);
     if (valid) {
-      const int page = tab[j / PAGE];
-      const T* kr = kpool + (((int64_t)page * G + g) * PAGE + (j % PAGE)) * DK;
+      const T* kr = kpool + (tile_row + lane) * DK;
       float x1 = 0.f, x2 = 0.f;
       if (vec8) {
         // 16-byte loads of 8 bf16 (rows are 16-byte aligned when D % 8 == 0)
@@ -130,12 +135,12 @@ __global__ __launch_bounds__(BLOCK) void diff_attn_row_kernel(
       a2[r] *= c2;
     }
     const int cnt = min(WAVE_SIZE, pos + 1 - j0);
+    const T* vtile = vpool + tile_row * V;
+#pragma unroll 8
     for (int jj = 0; jj < cnt; ++jj) {
       const float w1 = __shfl(p1, jj, WAVE_SIZE);
       const float w2 = __shfl(p2, jj, WAVE_SIZE);
-      const int jk = j0 + jj;
-      const int page = tab[jk / PAGE];
-      const T* vr = vpool + (((int64_t)page * G + g) * PAGE + (jk % PAGE)) * V;
+      const T* vr = vtile + (int64_t)jj * V;
 #pragma unroll
       for (int r = 0; r < VR; ++r) {
         const int c = lane + r * WAVE_SIZE;

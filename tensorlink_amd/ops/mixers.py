@@ -285,7 +285,7 @@ def diff_attention(q: torch.Tensor, q_off: int, kpool: torch.Tensor,
         # over several blocks so the chip is filled; a function of the
         # step's shape only
         n_split = 1
-        while (n_split < 16 and meta.T * H * n_split < 512
+        while (n_split < 16 and meta.T * H * n_split < 1024
                and meta.max_kv > 512 * n_split):
             n_split *= 2
         return _ext().diff_attn_rows(q, q_off, kpool, vpool, meta.tok_seq,
