@@ -1,7 +1,7 @@
 """Serving load benchmark: Poisson request arrivals against the
 continuous batcher; reports throughput and TTFT/TPOT percentiles.
 
-The reference ships no load-testing tool (SURVEY.md §6: it publishes no
+The reference ships no load-testing tool (it publishes no
 performance numbers at all); this is the vLLM-``benchmark_serving``-style
 harness for this engine. Runs the batcher directly (no HTTP overhead) —
 point it at a GPU box for real numbers, or at the CPU tier for a smoke:

@@ -1,6 +1,6 @@
 #!/bin/bash
 # First-GPU-hour validation sweep (ROADMAP item 7): run the whole GPU
-# tier, the serving load benchmark with every round-1 serving feature
+# tier, the serving load benchmark with every earlier serving feature
 # on, the big-model smokes, and a headline bench point. Run via:
 #   /usr/local/graft/bin/gpurun --timeout 3000 -- 'bash scripts/gpu_validate.sh'
 set -x

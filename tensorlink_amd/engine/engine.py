@@ -7,7 +7,7 @@ This is the MI355X collapse of the reference's validator serving machinery
 lifecycle 901-1103, demand tracking 181-260) plus the job table that
 replaces the DHT. Each generated token goes decode-loop -> queue -> SSE
 (the reference routes it GPU -> IPC -> TCP -> net thread -> IPC poll ->
-format -> IPC -> asyncio queue, SURVEY.md §3.3).
+format -> IPC -> asyncio queue).
 
 SPMD: rank 0 owns the engine API; ranks 1..N-1 sit in
 :meth:`InferenceEngine.worker_loop` executing broadcast commands.

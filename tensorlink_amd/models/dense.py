@@ -219,7 +219,7 @@ class MLP(nn.Module):
 
 class MoEMLP(nn.Module):
     """Mixtral-style sparse MoE block (new capability — the reference has no
-    MoE-aware code, SURVEY.md §2.2)."""
+    MoE-aware code)."""
 
     def __init__(self, config: ModelConfig):
         super().__init__()

@@ -1,7 +1,6 @@
 """GPT-NeoX / Pythia model family.
 
-Proves the zoo extends beyond the Llama shape (VERDICT r1 missing #2 —
-the reference auto-stages ANY HF causal LM via its AST injector,
+Proves the zoo extends beyond the Llama shape (the reference auto-stages ANY HF causal LM via its AST injector,
 ``tensorlink/ml/injector.py:79-90``): LayerNorm with bias (not RMSNorm),
 PARALLEL attention+MLP residual (x + attn(ln1 x) + mlp(ln2 x)), partial
 rotary embeddings (``rotary_pct`` of each head rotated, the rest passed

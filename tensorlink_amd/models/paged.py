@@ -1,7 +1,7 @@
 """Paged KV cache (vLLM-style block tables) for long-context serving.
 
-SURVEY.md §2.4/§5 names the paged-KV decode kernel as the long-context
-story: instead of one contiguous [B, Hkv, Smax, D] slab per sequence, K/V
+The paged-KV decode kernel is the long-context story: instead of one
+contiguous [B, Hkv, Smax, D] slab per sequence, K/V
 live in a shared pool of 128-position pages and a per-sequence block table
 maps position/128 -> page id. The decode and rope+append kernels take the
 table (decode_attn_mfma.hip / rope_append.hip, PAGED variants), so

@@ -161,7 +161,7 @@ def quantize_mxfp4(w: torch.Tensor, group: int = 32):
     """Quantize [N, K] weights to MXFP4: groups of 32 along K share one
     power-of-two e8m0 scale; elements are e2m1 (±{0,.5,1,1.5,2,3,4,6}),
     packed two per byte. This is the exact operand format of gfx950's
-    scaled-MFMA instructions (CDNA4 guide §MX), so round-2's 4-bit GEMM
+    scaled-MFMA instructions (CDNA4 guide §MX), so a 4-bit GEMM
     kernel consumes these tensors directly; until then Fp4Linear
     dequantizes on the fly. Returns (packed [N, K//2] uint8,
     exponents [N, K/group] int8)."""
@@ -198,7 +198,7 @@ def dequantize_mxfp4(packed: torch.Tensor, exponents: torch.Tensor,
 class Fp4Linear(nn.Module):
     """Weight-only MXFP4 linear: 4x smaller weights than bf16. Forward
     dequantizes per call (correct everywhere; the scaled-MFMA GEMM that
-    consumes the packed form directly is round-2 kernel work —
+    consumes the packed form directly is later kernel work —
     ROADMAP.md §6)."""
 
     def __init__(self, packed, exponents, bias, in_features, out_features):

@@ -220,7 +220,7 @@ def attention_prefill(q, k, v, causal: bool = True,
             and q.shape[1] == k.shape[1]):
         # long-context full prefill: ROCm flash SDPA measured faster
         # than the hand-written kernel at S >= 4k (376 vs 259 TF,
-        # profiles/ r1); chunked/q_off windows stay on the HIP kernel
+        # profiles/); chunked/q_off windows stay on the HIP kernel
         out = torch.nn.functional.scaled_dot_product_attention(
             q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2),
             is_causal=True, scale=scale, enable_gqa=True)

@@ -3,7 +3,7 @@
 // Replaces the reference's per-module torch.optim step executed on each
 // worker (tensorlink/ml/worker.py:1279-1297). The Python-side optimizer
 // flattens a stage's parameters into ONE contiguous buffer, so the whole
-// stage steps in a single launch (cf. SURVEY.md §2.1 "one fused HIP Adam
+// stage steps in a single launch (cf. the plan's "one fused HIP Adam
 // kernel launch per stage rank").
 //
 // param: bf16 or fp32 [n]; grad: same dtype as param; exp_avg/exp_avg_sq:

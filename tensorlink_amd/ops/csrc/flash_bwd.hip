@@ -1,7 +1,7 @@
 // Causal GQA flash-attention BACKWARD on gfx950 MFMA (training path).
 //
-// Replaces the round-1 torch-SDPA composition for training attention
-// (VERDICT r1 missing #5): two kernels recompute P from the forward's
+// Replaces the earlier torch-SDPA composition for training attention:
+// two kernels recompute P from the forward's
 // saved logsumexp and produce the three gradients:
 //
 //   dKV kernel — grid (kv_tiles, Hkv, B): a block owns 64 keys of one

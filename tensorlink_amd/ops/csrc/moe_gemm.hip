@@ -1,6 +1,6 @@
 // Grouped expert GEMM for MoE serving (gfx950).
 //
-// Replaces the per-expert Python loop (round-1 models/dense.py MoEMLP /
+// Replaces the per-expert Python loop (earlier models/dense.py MoEMLP /
 // models/quant.py): ONE launch computes out[p] = x[tok_idx[p]] @
 // W[e]^T for every (token, expert-slot) pair p, where pairs are sorted
 // by expert into segments (seg_off[e]..seg_off[e+1]). Expert weights

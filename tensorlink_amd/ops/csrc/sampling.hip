@@ -1,7 +1,7 @@
 // Fused on-device token sampling for serving decode (gfx950).
 //
 // The reference delegates sampling to HF generate()'s host-side logits
-// processors (SURVEY.md §2.4 row "LM head + sampling"); here the whole
+// processors (kernel-surface row "LM head + sampling"); here the whole
 // chain — presence/frequency penalties, temperature, top-k, top-p,
 // draw — runs in ONE kernel, one block per row, so sampled decode can
 // be captured in a hipGraph (counter-based RNG, no host RNG state).

@@ -1,5 +1,5 @@
 """Context (sequence) parallelism for prefill — ring attention (opt-in,
-beyond reference parity; SURVEY.md §2.2 lists SP/CP as a stretch goal).
+beyond reference parity; the survey lists SP/CP as a stretch goal).
 
 The sequence is sharded across ranks (weights replicated); each rank
 computes attention for its query chunk while K/V chunks rotate around the

@@ -1,7 +1,7 @@
 """Hybrid data-parallel × pipeline-parallel training.
 
 The reference plumbs a ``dp_factor`` through its job requests but never
-implements replication (``nodes/user_thread.py:139``, SURVEY.md §2.2 —
+implements replication (``nodes/user_thread.py:139`` —
 "Parameter only — NOT implemented"). Here DP is real: world = dp × pp,
 contiguous pipeline groups (adjacent stages stay on adjacent xGMI
 neighbors), and gradients are averaged across replicas with ONE RCCL

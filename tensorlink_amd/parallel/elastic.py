@@ -2,7 +2,7 @@
 
 The reference detects dead workers with heartbeat pings and drops them
 from the distributed graph but leaves re-forming to operator restart
-(``nodes/job_monitor.py`` health loop; SURVEY.md §2.6 "failure
+(``nodes/job_monitor.py`` health loop; "failure
 detection"). Here the survivors recover THEMSELVES: a collective that
 fails (peer socket closed / RCCL error) triggers a survivor rendezvous on
 a side TCPStore, the group re-initializes with the survivor count, the

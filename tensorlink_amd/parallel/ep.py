@@ -1,6 +1,6 @@
 """Expert parallelism for MoE layers (opt-in, beyond reference parity).
 
-The reference has no MoE-aware code at all (SURVEY.md §2.2); this build's
+The reference has no MoE-aware code at all; this build's
 default places each layer's full expert set on its pipeline stage. EP
 additionally shards the EXPERTS of every MoE layer across ranks: each
 rank stores and computes only its num_experts/ep local experts, the

@@ -1,6 +1,6 @@
 """Tensor parallelism (opt-in, beyond reference parity).
 
-The reference has no intra-layer sharding (SURVEY.md §2.2: "TP: NO").
+The reference has no intra-layer sharding ("TP: NO").
 This module adds Megatron-style TP for inference: attention heads and MLP
 intermediate are sharded column-parallel across ranks; the o/down
 projections are row-parallel and their outputs are summed with ONE RCCL

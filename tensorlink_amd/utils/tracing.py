@@ -2,7 +2,7 @@
 
 The reference has NO tracing subsystem — its closest artifacts are
 per-token ``time.time()`` deltas (``ml/formatter.py:353``) and ad-hoc GPU
-memory prints (``ml/worker.py:801-817``); SURVEY.md §5 makes a proper
+memory prints (``ml/worker.py:801-817``); the survey makes a proper
 profile path a deliverable of this build. Kernel-level timing comes from
 ``rocprofv3`` (see profiles/README.md); this module covers the layer the
 kernel profiler cannot see — engine phases (prefill, decode steps,

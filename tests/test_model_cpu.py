@@ -768,8 +768,8 @@ def test_lora_gpt2_defaults():
 
 def test_neox_family():
     """GPT-NeoX family: pp2 == pp1 generation, HF checkpoint loading
-    with qkv de-interleave, and from_hf_config mapping (VERDICT r1
-    missing #2 — a non-Llama-shaped architecture in the zoo)."""
+    with qkv de-interleave, and from_hf_config mapping (a
+    non-Llama-shaped architecture in the zoo)."""
     import json
     import tempfile
 

@@ -1,5 +1,5 @@
 """HIP kernel numerics tests (MI355X): each kernel vs a plain PyTorch fp32
-reference of the same op (SURVEY.md §4: the kernel-unit tier the reference
+reference of the same op (the kernel-unit tier the reference
 lacks; cf. its gradient-hash idea ml/proofs.py:6)."""
 
 import math
@@ -551,7 +551,7 @@ def test_moe_fused_block_matches_loop():
 
 def test_moe_fp8_graph_decode():
     """Quantized-MoE decode is hipGraph-captured with the grouped kernel
-    (round 1 disabled graphs for fp8 because of _scaled_mm)."""
+    (an earlier version disabled graphs for fp8 because of _scaled_mm)."""
     from tensorlink_amd.parallel.pipeline import PipelineRunner, SamplingParams
     from tensorlink_amd.parallel.planner import plan_for_world
     r = PipelineRunner(plan_for_world("tiny-moe", 1), 0, 1, device=DEV,

@@ -1372,7 +1372,7 @@ def _pp_compose_worker(rank, world, port, q):
 
 @pytest.mark.timeout(300)
 def test_pp2_spec_prefix_chunked_composition():
-    """The round-1 failing composition (chunked prefill + prefix caching
+    """The earlier failing composition (chunked prefill + prefix caching
     + speculation) on the PP batcher: repeat prompt reuses pages, the
     lockstep ragged verify accepts proposals, and output equals serial
     greedy."""

@@ -1,4 +1,4 @@
-"""RCCL-on-hardware coverage within a 1-GPU lease (VERDICT r1 item 5).
+"""RCCL-on-hardware coverage within a 1-GPU lease.
 
 RCCL refuses two ranks on one device ("Duplicate GPU detected", verified
 on MI355X — the communicator requires distinct devices), so a single
