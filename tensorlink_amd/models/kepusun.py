@@ -119,11 +119,12 @@ class KepusunLayer(nn.Module):
         self.mlp = None
         if mlp is not None:
             r = mlp["router"]
+            groups = r.get("groups") or {"count": 1, "keep": 1}
             self.norm2 = DynamicTanh(w)
             self.hc2 = HyperConnection(ns)
             self.mlp = GroupLimitedMoE(w, mlp["expert"]["ff"], r["experts"],
-                                       r["top"], r["groups"]["count"],
-                                       r["groups"]["keep"], r["scale"])
+                                       r["top"], groups["count"],
+                                       groups["keep"], r.get("scale", 1.0))
 
 
 class KepusunStageModel(nn.Module):
@@ -314,6 +315,12 @@ def load_kepusun_weights(stage: KepusunStageModel, ckpt_dir: str,
             filled[pname] += t.numel()
             loaded += 1
     short = [k for k, n in filled.items() if n != P[k].numel()]
+    if stage.config.streams == 1:
+        # a single stream without hyper-connection tensors is the plain
+        # pre-norm residual: the identity defaults stand
+        short = [k for k in short
+                 if not (filled[k] == 0 and k.rsplit(".", 1)[-1]
+                         in ("inw", "out", "mix") and ".hc" in k)]
     if short:
         raise KeyError(f"checkpoint leaves parameters unfilled: {short[:5]}")
     return loaded

@@ -613,3 +613,21 @@ def test_config_and_loader_are_strict(tmp_path):
     write_checkpoint(d3, cfg2, P)
     with pytest.raises(KeyError):
         get_config(d3)
+
+
+def test_single_stream_without_hyper_connection_tensors(tmp_path):
+    """One stream and no hc tensors in the checkpoint is the plain
+    pre-norm residual x + f(norm(x))."""
+    cfg = cfg_ones()
+    P = make_weights(cfg, seed=3)
+    for k in list(P):
+        if ".hc" in k:
+            P[k] = torch.ones_like(P[k])
+    d = str(tmp_path / "m")
+    write_checkpoint(d, cfg, {k: v for k, v in P.items() if ".hc" not in k})
+    runner = PipelineRunner(plan_for_world(d, 1), 0, 1,
+                            device=torch.device("cpu"), init="checkpoint",
+                            ckpt_dir=d, dtype=torch.float32)
+    toks = tokens(cfg, 40, 9)
+    got = run_schedule(batcher(runner), toks, [17, 2])
+    assert close(got, oracle(toks, P, cfg), torch.float32)
