@@ -454,4 +454,7 @@ def _stage_class(config: ModelConfig):
     if config.architecture == "kepusun":
         from tensorlink_amd.models.kepusun import KepusunStageModel
         return KepusunStageModel
+    if config.architecture == "senulix":
+        from tensorlink_amd.models.senulix import SenulixStageModel
+        return SenulixStageModel
     return StageModel

@@ -26,6 +26,7 @@ import torch.nn as nn
 
 from tensorlink_amd.models.configs import ModelConfig
 from tensorlink_amd.models.dense import TLLinear
+from tensorlink_amd.models.layered import LayeredStage, load_named_tensors
 from tensorlink_amd.models.mixers import (DiffAttention, DynamicTanh,
                                           GroupLimitedMoE, HyperConnection,
                                           MLSTMMixer)
@@ -127,11 +128,8 @@ class KepusunLayer(nn.Module):
                                        groups["keep"], r.get("scale", 1.0))
 
 
-class KepusunStageModel(nn.Module):
+class KepusunStageModel(LayeredStage):
     """Whole-model stage (embedding, every layer, final norm + head)."""
-
-    SUPPORTS_RAGGED = True      # one forward serves a mixed ragged batch
-    GRAPH_CAPTURE = False       # host-built ragged metadata every step
 
     def __init__(self, config: KepusunConfig, layer_start: int,
                  layer_end: int, has_embedding: bool, has_head: bool):
@@ -153,39 +151,7 @@ class KepusunStageModel(nn.Module):
                                 bias=False)
         self.layer_sums = None      # list -> per-layer stream sums (debug)
 
-    @property
-    def num_layers(self):
-        return len(self.layers)
-
-    # ---------------------------------------------------------- cache
-    def cache_specs(self):
-        return [l.mix.cache_spec() for l in self.layers]
-
-    def make_slot_cache(self, slots: int, pool_pages: int, max_seq: int,
-                        device, dtype):
-        from tensorlink_amd.models.paged import HybridSlotCache
-        return HybridSlotCache(self.cache_specs(), slots, pool_pages,
-                               max_seq, device, dtype)
-
-    def make_kv_cache(self, batch: int, max_seq: int, device, dtype=None,
-                      kv_mode: str = "paged"):
-        """Rectangular-batch cache for ``PipelineRunner.generate``: one
-        slot per row with its pages leased up front."""
-        from tensorlink_amd.models.paged import PAGE
-        if dtype is None:
-            dtype = self.lm_head.weight.dtype
-        pps = (max_seq + PAGE - 1) // PAGE
-        cache = self.make_slot_cache(batch, batch * pps, max_seq, device,
-                                     dtype)
-        for s in range(batch):
-            cache.ensure(s, max_seq)
-        cache.static = True
-        return cache
-
     # -------------------------------------------------------- forward
-    def embed(self, input_ids):
-        return self.embed_tokens(input_ids)
-
     def head(self, hidden: torch.Tensor) -> torch.Tensor:
         """Final Dynamic-Tanh norm + vocabulary projection of summed
         streams [..., W] (fp32)."""
@@ -194,18 +160,6 @@ class KepusunStageModel(nn.Module):
         h, _ = mx.hyper_dyt(X, None, None, None, None, *self.norm.params(),
                             out_dtype=self.lm_head.weight.dtype)
         return self.lm_head(h).reshape(*shape[:-1], -1)
-
-    def _meta(self, kv_cache, positions, B, S):
-        meta = getattr(kv_cache, "ragged", None)
-        if meta is not None:
-            return meta
-        # rectangular batch: B sequences of S new tokens each
-        pos0 = positions.reshape(B, S)[:, 0].tolist()
-        slots = getattr(kv_cache, "slot_ids", None)
-        if slots is None:
-            slots = list(range(B))
-        return mx.RaggedMeta([S] * B, pos0, slots, kv_cache.table[:B],
-                             positions.device)
 
     @torch.no_grad()
     def forward(self, hidden_or_ids, positions, kv_cache=None,
@@ -294,36 +248,14 @@ def load_kepusun_weights(stage: KepusunStageModel, ckpt_dir: str,
                          dtype=torch.bfloat16) -> int:
     """Fill the stage from ``model.safetensors``; every tensor of the
     checkpoint must be consumed and every parameter filled."""
-    from safetensors import safe_open
     names, P = _name_map(stage)
-    filled = {k: 0 for k in P}
-    loaded = 0
-    with safe_open(os.path.join(ckpt_dir, "model.safetensors"),
-                   framework="pt", device="cpu") as f:
-        for key in f.keys():
-            if key not in names:
-                raise KeyError(f"unexpected tensor {key!r} in checkpoint")
-            pname, off = names[key]
-            t = f.get_tensor(key)
-            p = P[pname]
-            if p.dim() == 0:
-                p.copy_(t.reshape(()))
-            elif p.dim() == 3:                      # stacked experts
-                p[off].copy_(t)
-            else:
-                p[off:off + t.shape[0]].copy_(t)
-            filled[pname] += t.numel()
-            loaded += 1
-    short = [k for k, n in filled.items() if n != P[k].numel()]
+    optional = []
     if stage.config.streams == 1:
         # a single stream without hyper-connection tensors is the plain
         # pre-norm residual: the identity defaults stand
-        short = [k for k in short
-                 if not (filled[k] == 0 and k.rsplit(".", 1)[-1]
-                         in ("inw", "out", "mix") and ".hc" in k)]
-    if short:
-        raise KeyError(f"checkpoint leaves parameters unfilled: {short[:5]}")
-    return loaded
+        optional = [k for k in P if ".hc" in k
+                    and k.rsplit(".", 1)[-1] in ("inw", "out", "mix")]
+    return load_named_tensors(P, names, ckpt_dir, optional)
 
 
 @torch.no_grad()

@@ -127,6 +127,11 @@ def load_stage_from_checkpoint(stage: StageModel, ckpt_dir: str,
         n = load_kepusun_weights(stage, ckpt_dir, dtype=dtype)
         stage.to(device=device, dtype=dtype)
         return n
+    if arch == "senulix":
+        from tensorlink_amd.models.senulix import load_senulix_weights
+        n = load_senulix_weights(stage, ckpt_dir, dtype=dtype)
+        stage.to(device=device, dtype=dtype)
+        return n
     from safetensors import safe_open
 
     index_path = os.path.join(ckpt_dir, "model.safetensors.index.json")
@@ -169,6 +174,10 @@ def init_random_stage(stage: StageModel, device="cpu", dtype=torch.bfloat16,
     if stage.config.architecture == "kepusun":
         from tensorlink_amd.models.kepusun import init_kepusun_random
         init_kepusun_random(stage, seed=seed)
+        return stage.to(device=device, dtype=dtype)
+    if stage.config.architecture == "senulix":
+        from tensorlink_amd.models.senulix import init_senulix_random
+        init_senulix_random(stage, seed=seed)
         return stage.to(device=device, dtype=dtype)
     gen_dev = device if str(device).startswith("cuda") else "cpu"
     g = torch.Generator(device=gen_dev)

@@ -235,3 +235,230 @@ class GroupLimitedMoE(nn.Module, _F32Cache):
             out.index_add_(0, tok, F.linear(a, self.down[e]).float()
                            * w[tok, choice, None])
         return out.to(h.dtype)
+
+
+# ---------------------------------------------------------------------------
+# blocks of the post-norm layered family: lightning (decayed linear)
+# attention, latent attention, windowed attention with score mixing and a
+# sink, plain two-matrix feed-forward, per-layer token input
+# ---------------------------------------------------------------------------
+class RMSWeight(nn.Module, _F32Cache):
+    """Weight of an RMS norm; ``one_plus`` = stored around zero and
+    applied as (1 + w)."""
+
+    def __init__(self, width: int, one_plus: bool):
+        super().__init__()
+        self.one_plus = bool(one_plus)
+        self.weight = nn.Parameter(torch.zeros(width) if one_plus
+                                   else torch.ones(width))
+
+    def w32(self):
+        return self._f32("weight")
+
+
+class LightningMixer(nn.Module, _F32Cache):
+    """Linear attention with one fixed decay per head: fused q|k|v|g
+    projection, silu on q, k, v, the slot-state recurrence
+    S <- decay S + k v^T, read-out S^T q, one RMS norm over all heads
+    together, sigmoid output gate, output projection."""
+
+    kind = "lightning"
+
+    def __init__(self, width: int, heads: int, dim: int, vdim: int,
+                 decay, eps: float):
+        super().__init__()
+        assert len(decay) == heads
+        self.H, self.D, self.V, self.eps = heads, dim, vdim, float(eps)
+        hd, hv = heads * dim, heads * vdim
+        self.offs = (0, hd, 2 * hd, 2 * hd + hv)
+        self.proj = TLLinear(width, 2 * hd + 2 * hv, bias=False)
+        self.norm = nn.Parameter(torch.ones(hv))
+        self.o_proj = TLLinear(hv, width, bias=False)
+        self.register_buffer("decay", torch.tensor(
+            [float(x) for x in decay], dtype=torch.float64),
+            persistent=False)
+
+    def cache_spec(self):
+        return {"kind": "state", "shapes": [(self.H, self.D, self.V)]}
+
+    def _decay32(self, dev):
+        hit = self.__dict__.get("_dec")
+        if hit is None or hit.device != dev:
+            hit = self.decay.to(device=dev, dtype=torch.float32)
+            self.__dict__["_dec"] = hit
+        return hit
+
+    def forward(self, h, meta, cache, layer_idx):
+        proj = self.proj(h)
+        (S,) = cache.state[layer_idx]
+        o = mx.lightning_scan(proj, self.offs[:3], self._decay32(h.device),
+                              S, meta, self.H, self.D, self.V)
+        y = mx.rms_scale(o, self._f32("norm"), self.eps, False, gate=proj,
+                         gate_col=self.offs[3], out_dtype=h.dtype)
+        return self.o_proj(y)
+
+
+class LatentAttention(nn.Module, _F32Cache):
+    """Attention whose cache holds, per token, one normed latent c
+    [kv_rank] and one rotated key part [rot_dim] shared by all heads.
+
+    Keys and values are linear in c (k_h = W_uk,h c, v_h = W_uv,h c), so
+    the heads' unrotated queries are carried into latent space
+    (q'_h = W_uk,h^T q_h) and every head attends the SAME cached rows
+    [c | k_rot] (one shared key head, values = the first kv_rank columns
+    of the row); W_uv is applied to the attended latent afterwards. The
+    per-head keys and values are never materialised. ``kv_from`` = index
+    of an earlier latent layer whose cached rows this layer reads with its
+    own W_uk / W_uv and queries."""
+
+    kind = "latent_attention"
+
+    def __init__(self, width: int, heads: int, dim: int, rot_dim: int,
+                 vdim: int, kv_rank: int, scale: float, rot_base: float,
+                 eps: float, kv_from: Optional[int] = None):
+        super().__init__()
+        assert rot_dim % 2 == 0
+        self.H, self.D, self.RD, self.V, self.R = (heads, dim, rot_dim, vdim,
+                                                   kv_rank)
+        self.scale, self.eps, self.base = float(scale), float(eps), rot_base
+        self.kv_from = kv_from
+        self.q_cols = heads * (dim + rot_dim)
+        self.kv_cols = 0 if kv_from is not None else kv_rank + rot_dim
+        self.qdkv = TLLinear(width, self.q_cols + self.kv_cols, bias=False)
+        if kv_from is None:
+            self.dkv_norm = nn.Parameter(torch.ones(kv_rank))
+        self.uk = nn.Parameter(torch.zeros(heads * dim, kv_rank))
+        self.uv = nn.Parameter(torch.zeros(heads * vdim, kv_rank))
+        self.o_proj = TLLinear(heads * vdim, width, bias=False)
+
+    def cache_spec(self):
+        if self.kv_from is not None:
+            return {"kind": "kv_ref", "src": self.kv_from}
+        return {"kind": "kv", "G": 1, "DK": self.R + self.RD, "V": 0}
+
+    def _freqs(self, dev):
+        hit = self.__dict__.get("_fr")
+        if hit is None or hit.device != dev:
+            hit = mx.rope_freqs(self.RD, self.base, dev)
+            self.__dict__["_fr"] = hit
+        return hit
+
+    def forward(self, h, meta, cache, layer_idx):
+        H, D, RD, R, V = self.H, self.D, self.RD, self.R, self.V
+        T = h.shape[0]
+        proj = self.qdkv(h)
+        fr = self._freqs(h.device)
+        src = layer_idx if self.kv_from is None else self.kv_from
+        pool = cache.k[src]
+        if self.kv_from is None:
+            mx.norm_rope_rows(proj, self.q_cols, 1, R + RD, meta,
+                              norm_w=self._f32("dkv_norm"), norm_cols=R,
+                              eps=self.eps, rot_off=R, rot_dims=RD,
+                              freqs=fr, pool=pool)
+        q = mx.norm_rope_rows(proj, 0, H, D + RD, meta, rot_off=D,
+                              rot_dims=RD, freqs=fr).view(T, H, D + RD)
+        qa = torch.empty(T, H, R + RD, device=h.device, dtype=torch.float32)
+        qa[:, :, R:] = q[:, :, D:]
+        torch.bmm(q[:, :, :D].transpose(0, 1),
+                  self._f32("uk").view(H, D, R),
+                  out=qa[:, :, :R].transpose(0, 1))
+        o = mx.flex_attention(qa.view(T, H * (R + RD)), pool, None, meta, H,
+                              self.scale, v_cols=R)
+        o = torch.bmm(o.view(T, H, R).transpose(0, 1),
+                      self._f32("uv").view(H, V, R).transpose(1, 2))
+        return self.o_proj(o.transpose(0, 1).reshape(T, H * V).to(h.dtype))
+
+
+class WindowAttention(nn.Module, _F32Cache):
+    """Grouped-query softmax attention over the paged pool with: one RMS
+    norm over the WHOLE query projection and one over the whole key
+    projection (plain weights, before rotation); rotate-half positions on
+    the first ``rot_dims`` dimensions of every head; a learned [H, H]
+    mixing of the heads' scores before the softmax (``talk``); a sliding
+    window (``window`` = 0: plain causal); a sink (one added to the
+    softmax denominator)."""
+
+    kind = "attention"
+
+    def __init__(self, width: int, heads: int, kv_heads: int, dim: int,
+                 vdim: int, scale: float, rot_dims: int, rot_base: float,
+                 window: int, eps: float, sink: bool = True,
+                 talk: bool = True, qk_norm: bool = True):
+        super().__init__()
+        assert heads % kv_heads == 0 and rot_dims % 2 == 0 and rot_dims <= dim
+        self.H, self.G, self.D, self.V = heads, kv_heads, dim, vdim
+        self.scale, self.eps = float(scale), float(eps)
+        self.rot_dims, self.base = int(rot_dims), rot_base
+        self.window, self.sink = int(window), bool(sink)
+        self.q_cols, self.k_cols = heads * dim, kv_heads * dim
+        self.qkv = TLLinear(width, self.q_cols + self.k_cols
+                            + kv_heads * vdim, bias=False)
+        self.q_norm = nn.Parameter(torch.ones(self.q_cols)) if qk_norm \
+            else None
+        self.k_norm = nn.Parameter(torch.ones(self.k_cols)) if qk_norm \
+            else None
+        self.talk = nn.Parameter(torch.eye(heads)) if talk else None
+        self.o_proj = TLLinear(heads * vdim, width, bias=False)
+
+    def cache_spec(self):
+        return {"kind": "kv", "G": self.G, "DK": self.D, "V": self.V}
+
+    def _freqs(self, dev):
+        hit = self.__dict__.get("_fr")
+        if hit is None or hit.device != dev:
+            hit = mx.rope_freqs(self.rot_dims, self.base, dev)
+            self.__dict__["_fr"] = hit
+        return hit
+
+    def forward(self, h, meta, cache, layer_idx):
+        proj = self.qkv(h)
+        fr = self._freqs(h.device) if self.rot_dims else None
+        qn = self._f32("q_norm") if self.q_norm is not None else None
+        kn = self._f32("k_norm") if self.k_norm is not None else None
+        kpool, vpool = cache.k[layer_idx], cache.v[layer_idx]
+        mx.norm_rope_rows(proj, self.q_cols, self.G, self.D, meta,
+                          norm_w=kn, norm_cols=self.k_cols, eps=self.eps,
+                          rot_dims=self.rot_dims, freqs=fr, pool=kpool)
+        mx.norm_rope_rows(proj, self.q_cols + self.k_cols, self.G, self.V,
+                          meta, pool=vpool)
+        q = mx.norm_rope_rows(proj, 0, self.H, self.D, meta, norm_w=qn,
+                              norm_cols=self.q_cols, eps=self.eps,
+                              rot_dims=self.rot_dims, freqs=fr)
+        o = mx.flex_attention(
+            q, kpool, vpool, meta, self.H, self.scale, window=self.window,
+            sink=self.sink,
+            talk=self._f32("talk") if self.talk is not None else None,
+            out_dtype=h.dtype)
+        return self.o_proj(o)
+
+
+class DenseFF(nn.Module):
+    """down(gelu(up x)), exact (erf) or tanh-form GELU, no biases."""
+
+    def __init__(self, width: int, ff: int, tanh_form: bool = False):
+        super().__init__()
+        self.tanh_form = bool(tanh_form)
+        self.up = TLLinear(width, ff, bias=False)
+        self.down = TLLinear(ff, width, bias=False)
+
+    def forward(self, h):
+        return self.down(mx.gelu(self.up(h), self.tanh_form))
+
+
+class TokenSide(nn.Module):
+    """Per-layer token input: a slice of a second embedding table gates a
+    narrow projection of the residual,
+    y = proj(gelu_tanh(gate x) * table[token, col:col + dim]); the caller
+    adds y through an RMS norm with the plain weight ``norm``."""
+
+    def __init__(self, width: int, dim: int, col: int):
+        super().__init__()
+        self.dim, self.col = dim, col
+        self.gate = TLLinear(width, dim, bias=False)
+        self.proj = TLLinear(dim, width, bias=False)
+        self.norm = RMSWeight(width, one_plus=False)
+
+    def forward(self, h, table, tokens):
+        g = mx.gelu(self.gate(h), True, table=table, tokens=tokens,
+                    table_col=self.col)
+        return self.proj(g)

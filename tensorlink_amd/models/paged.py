@@ -154,11 +154,14 @@ class HybridSlotCache(DynamicPagedKVCache):
     earlier layer's pools (cross-layer KV sharing), or fp32 recurrent
     state indexed by slot.
 
-    ``specs[l]`` is ``{"kind": "kv", "G", "DK", "V"}``,
-    ``{"kind": "kv_ref", "src": j}`` or ``{"kind": "mlstm", "H", "D",
-    "V"}``. ``k[l]`` / ``v[l]`` are [pool_pages, G, PAGE, DK|V] (None for
-    recurrent layers, the source's tensors for references); ``state[l]``
-    is (S [slots, H, D, V], n [slots, H, D], m [slots, H]) or None. Pages
+    ``specs[l]`` is ``{"kind": "kv", "G", "DK", "V"}`` (``V`` = 0: key
+    rows only, for layers whose values are part of the key row),
+    ``{"kind": "kv_ref", "src": j}``, ``{"kind": "mlstm", "H", "D",
+    "V"}`` or ``{"kind": "state", "shapes": [...]}``. ``k[l]`` / ``v[l]``
+    are [pool_pages, G, PAGE, DK|V] (None for recurrent layers, the
+    source's tensors for references); ``state[l]`` is (S [slots, H, D, V],
+    n [slots, H, D], m [slots, H]) for ``mlstm``, one fp32 tensor
+    [slots, *shape] per entry of ``shapes`` for ``state``, else None. Pages
     are leased and returned exactly as in :class:`DynamicPagedKVCache`;
     recurrent state needs no clearing on release because the kernels start
     a sequence with no cached tokens from zeros."""
@@ -176,12 +179,19 @@ class HybridSlotCache(DynamicPagedKVCache):
                                           dtype=dtype))
                 self.v.append(torch.zeros(pool_pages, sp["G"], PAGE,
                                           sp["V"], device=device,
-                                          dtype=dtype))
+                                          dtype=dtype) if sp["V"] else None)
                 self.state.append(None)
             elif sp["kind"] == "kv_ref":
                 self.k.append(self.k[sp["src"]])
                 self.v.append(self.v[sp["src"]])
                 self.state.append(None)
+            elif sp["kind"] == "state":
+                self.k.append(None)
+                self.v.append(None)
+                self.state.append(tuple(
+                    torch.zeros(slots, *shape, device=device,
+                                dtype=torch.float32)
+                    for shape in sp["shapes"]))
             else:
                 f32 = dict(device=device, dtype=torch.float32)
                 self.k.append(None)

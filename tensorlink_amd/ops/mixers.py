@@ -344,3 +344,225 @@ def group_limited_router(logits: torch.Tensor, top: int, n_groups: int,
     w = s.gather(1, idx)
     w = w / (w.sum(-1, keepdim=True) + 1e-20) * scale
     return w, idx
+
+
+# ---------------------------------------------------------------------------
+# post-norm residual, gated / plain RMS scaling, GELU, soft cap
+# ---------------------------------------------------------------------------
+def _rms(x: torch.Tensor, eps: float) -> torch.Tensor:
+    return x * torch.rsqrt((x * x).mean(-1, keepdim=True) + eps)
+
+
+def postnorm_add(X: torch.Tensor, y: torch.Tensor, w: torch.Tensor,
+                 eps: float, one_plus: bool, out_dtype=torch.float32):
+    """Residual with the norm on the sublayer's OUTPUT, in place on the
+    fp32 residual X [T, W]:  X += y / rms(y) * (1 + w  |  w).
+    Returns X in ``out_dtype`` (the next sublayer's input; X itself for
+    fp32)."""
+    assert X.dtype == torch.float32 and w.dtype == torch.float32
+    if X.is_cuda:
+        return _ext().postnorm_add(X, y.contiguous(), w, float(eps),
+                                   bool(one_plus),
+                                   out_dtype == torch.float32)
+    X += _rms(y.float(), eps) * ((1.0 + w) if one_plus else w)
+    return X if out_dtype == torch.float32 else X.to(out_dtype)
+
+
+def rms_scale(x: torch.Tensor, w: torch.Tensor, eps: float, one_plus: bool,
+              gate: Optional[torch.Tensor] = None, gate_col: int = 0,
+              out_dtype=torch.float32) -> torch.Tensor:
+    """x / rms(x) * (1 + w | w) over the last axis of x [T, N] (fp32),
+    optionally times sigmoid(gate[:, gate_col:gate_col + N])."""
+    assert x.dtype == torch.float32 and w.dtype == torch.float32
+    if x.is_cuda:
+        return _ext().rms_scale(x.contiguous(), w, float(eps),
+                                bool(one_plus), gate, int(gate_col),
+                                out_dtype == torch.float32)
+    y = _rms(x, eps) * ((1.0 + w) if one_plus else w)
+    if gate is not None:
+        y = y * torch.sigmoid(
+            gate[:, gate_col:gate_col + x.shape[-1]].float())
+    return y.to(out_dtype)
+
+
+def gelu(x: torch.Tensor, tanh_form: bool = False,
+         table: Optional[torch.Tensor] = None,
+         tokens: Optional[torch.Tensor] = None,
+         table_col: int = 0) -> torch.Tensor:
+    """GELU of x [T, N] — exact (erf) or the tanh form — evaluated in fp32,
+    optionally times ``table[tokens, table_col:table_col + N]`` (a
+    per-token embedding slice gathered in the same pass)."""
+    if x.is_cuda:
+        return _ext().gelu_mul(x.contiguous(), bool(tanh_form), table,
+                               tokens, int(table_col))
+    y = torch.nn.functional.gelu(x.float(),
+                                 approximate="tanh" if tanh_form else "none")
+    if table is not None:
+        y = y * table[tokens.long(),
+                      table_col:table_col + x.shape[-1]].float()
+    return y.to(x.dtype)
+
+
+def soft_cap_(z: torch.Tensor, cap: float) -> torch.Tensor:
+    """cap * tanh(z / cap) in place on fp32 logits."""
+    assert z.dtype == torch.float32
+    if z.is_cuda:
+        _ext().soft_cap_(z, float(cap))
+        return z
+    return z.copy_(cap * torch.tanh(z / cap))
+
+
+# ---------------------------------------------------------------------------
+# row preparation: RMS norm over a projection + rotate-half positions,
+# written densely (queries) or into a page pool (keys, values, latents)
+# ---------------------------------------------------------------------------
+def rope_freqs(dims: int, base: float, device) -> torch.Tensor:
+    """f_i = base^(-2i/dims), i < dims/2, evaluated in float64 and kept
+    there (the angle p * f_i is formed in double by the kernels)."""
+    i = torch.arange(dims // 2, dtype=torch.float64)
+    return torch.pow(torch.tensor(float(base), dtype=torch.float64),
+                     -2.0 * i / dims).to(device)
+
+
+def norm_rope_rows(src: torch.Tensor, col: int, n_heads: int, head_dim: int,
+                   meta: RaggedMeta, *, norm_w: Optional[torch.Tensor] = None,
+                   norm_cols: int = 0, eps: float = 0.0, rot_off: int = 0,
+                   rot_dims: int = 0, freqs: Optional[torch.Tensor] = None,
+                   pool: Optional[torch.Tensor] = None):
+    """Take columns [col, col + n_heads*head_dim) of src [T, L]; RMS-norm
+    the first ``norm_cols`` of them together (weight ``norm_w``, plain);
+    rotate dims [rot_off, rot_off + rot_dims) of every head by the token's
+    position (pairs (i, i + rot_dims/2), angle pos * freqs[i]); all in
+    fp32. Without ``pool`` returns the rows as fp32 [T, n_heads*head_dim];
+    with ``pool`` [pages, n_heads, PAGE, head_dim] scatters them to the
+    tokens' page rows in the pool's dtype and returns None."""
+    N = n_heads * head_dim
+    T = src.shape[0]
+    if src.is_cuda:
+        out = None if pool is not None else torch.empty(
+            T, N, device=src.device, dtype=torch.float32)
+        _ext().norm_rope_rows(src, int(col), int(n_heads), int(head_dim),
+                              norm_w, int(norm_cols), float(eps),
+                              int(rot_off), int(rot_dims), freqs,
+                              meta.tok_seq, meta.tok_pos, meta.table, out,
+                              pool)
+        return out
+    x = src[:, col:col + N].float()
+    if norm_w is not None:
+        x = torch.cat([_rms(x[:, :norm_cols], eps) * norm_w,
+                       x[:, norm_cols:]], 1)
+    x = x.reshape(T, n_heads, head_dim).clone()
+    pos = meta.tok_pos.long()
+    if rot_dims:
+        half = rot_dims // 2
+        ang = pos.double().view(T, 1, 1) * freqs.double().view(1, 1, half)
+        c, s = torch.cos(ang).float(), torch.sin(ang).float()
+        u = x[:, :, rot_off:rot_off + half].clone()
+        v = x[:, :, rot_off + half:rot_off + rot_dims].clone()
+        x[:, :, rot_off:rot_off + half] = u * c - v * s
+        x[:, :, rot_off + half:rot_off + rot_dims] = v * c + u * s
+    if pool is None:
+        return x.reshape(T, N)
+    page = meta.table.long()[meta.tok_seq.long(), pos // PAGE]
+    pool[page, :, pos % PAGE] = x.to(pool.dtype)
+    return None
+
+
+# ---------------------------------------------------------------------------
+# softmax attention over the paged pool with the options layered models
+# combine: GQA/MQA, sliding window, sink, cross-head score mixing, values
+# that are a prefix of the key row (latent attention)
+# ---------------------------------------------------------------------------
+def flex_attention(q: torch.Tensor, kpool: torch.Tensor,
+                   vpool: Optional[torch.Tensor], meta: RaggedMeta, H: int,
+                   scale: float, *, window: int = 0, sink: bool = False,
+                   talk: Optional[torch.Tensor] = None, v_cols: int = 0,
+                   out_dtype=torch.float32) -> torch.Tensor:
+    """Causal attention of the step's tokens over their sequences' cached
+    rows (the step's own rows already appended).
+
+    q [T, H*DK] fp32 (normed / rotated); kpool [pages, G, PAGE, DK];
+    values from vpool [pages, G, PAGE, V], or, without it, the first
+    ``v_cols`` columns of the key row. score = q.k * scale; with ``talk``
+    [H, H] the heads' scores are mixed, s_h <- sum_g talk[h, g] s_g;
+    ``window`` > 0 keeps keys with 0 <= i - j < window; ``sink`` adds one
+    to the softmax denominator. Scores, weights and sums are fp32.
+    Returns [T, H*V] in ``out_dtype``."""
+    G, DK = kpool.shape[1], kpool.shape[3]
+    V = vpool.shape[3] if vpool is not None else v_cols
+    T = q.shape[0]
+    assert q.dtype == torch.float32 and q.shape[1] == H * DK
+    if q.is_cuda:
+        return _ext().flex_attn_rows(q, kpool, vpool, meta.tok_seq,
+                                     meta.tok_pos, meta.table, talk, int(H),
+                                     float(scale), int(window), bool(sink),
+                                     int(V), out_dtype == torch.float32)
+    out = torch.empty(T, H, V)
+    qf = q.view(T, H, DK)
+    rep = H // G
+    for b in range(meta.B):
+        t0, t1 = meta.cu_h[b], meta.cu_h[b + 1]
+        if t1 == t0:
+            continue
+        L = meta.pos0_h[b] + (t1 - t0)
+        pages = meta.table[b, :(L + PAGE - 1) // PAGE].long()
+        kb = kpool[pages].float().permute(0, 2, 1, 3).reshape(-1, G, DK)[:L]
+        vb = (vpool[pages].float().permute(0, 2, 1, 3).reshape(-1, G, V)[:L]
+              if vpool is not None else kb[:, :, :V])
+        kb = kb.repeat_interleave(rep, 1)                 # [L, H, DK]
+        vb = vb.repeat_interleave(rep, 1)
+        sc = torch.einsum("thd,jhd->htj", qf[t0:t1], kb) * scale
+        if talk is not None:
+            sc = torch.einsum("hg,gtj->htj", talk.float(), sc)
+        qpos = torch.arange(meta.pos0_h[b], L).view(-1, 1)
+        kpos = torch.arange(L).view(1, -1)
+        hide = kpos > qpos
+        if window > 0:
+            hide = hide | (qpos - kpos >= window)
+        sc = sc.masked_fill(hide, float("-inf"))
+        m = sc.amax(-1, keepdim=True)
+        if sink:
+            m = m.clamp_min(0.0)
+        e = torch.exp(sc - m)
+        den = e.sum(-1, keepdim=True)
+        if sink:
+            den = den + torch.exp(-m)
+        out[t0:t1] = torch.einsum("htj,jhv->thv", e / den, vb)
+    return out.reshape(T, H * V).to(out_dtype)
+
+
+# ---------------------------------------------------------------------------
+# lightning attention: decayed outer-product memory per head
+# ---------------------------------------------------------------------------
+def lightning_scan(proj: torch.Tensor, offs, decay: torch.Tensor,
+                   S: torch.Tensor, meta: RaggedMeta, H: int, D: int,
+                   V: int) -> torch.Tensor:
+    """S_t = decay_h S_(t-1) + k_t v_t^T,  o_t = S_t^T q_t  per head, with
+    q, k, v = silu of columns ``offs`` = (q, k, v) of proj [T, L]. The
+    state pool S [slots, H, D, V] (fp32) is read at ``meta.slots`` (zeros
+    for a sequence with no cached tokens) and written back. Returns the
+    raw read-out [T, H*V] in fp32."""
+    q_off, k_off, v_off = offs
+    T = proj.shape[0]
+    if proj.is_cuda:
+        return _ext().lightning_scan(proj, int(q_off), int(k_off),
+                                     int(v_off), decay, S, meta.cu,
+                                     meta.slots, meta.pos0, int(H), int(D),
+                                     int(V))
+    silu = torch.nn.functional.silu
+    pf = proj.float()
+    q = silu(pf[:, q_off:q_off + H * D]).view(T, H, D)
+    k = silu(pf[:, k_off:k_off + H * D]).view(T, H, D)
+    v = silu(pf[:, v_off:v_off + H * V]).view(T, H, V)
+    o = torch.empty(T, H, V)
+    dec = decay.float().view(H, 1, 1)
+    for b in range(meta.B):
+        slot = meta.slots_h[b]
+        Sb = (torch.zeros(H, D, V) if meta.pos0_h[b] == 0
+              else S[slot].clone())
+        for t in range(meta.cu_h[b], meta.cu_h[b + 1]):
+            Sb = dec * Sb + k[t].unsqueeze(-1) * v[t].unsqueeze(-2)
+            o[t] = (Sb * q[t].unsqueeze(-1)).sum(1)
+        if meta.new_h[b] > 0:
+            S[slot] = Sb
+    return o.reshape(T, H * V)
