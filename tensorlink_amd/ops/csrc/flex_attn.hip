@@ -1,0 +1,416 @@
+// Softmax attention over a paged pool with the options that layered
+// models combine (gfx950): grouped / single key heads, sliding window,
+// a sink in the denominator, mixing of the heads' scores before the
+// softmax, and values that are a prefix of the key row (latent attention,
+// where every head attends the same cached rows [latent | rotated key]).
+//
+// tl_norm_rope_rows prepares rows of a fused projection: one RMS norm over
+// a leading range of the columns (the WHOLE query or key projection, or
+// the latent part of a latent row), rotate-half positions on a sub-range of
+// every head, then either a dense fp32 copy (queries) or a scatter into the
+// tokens' page rows (keys, values, latents). Angles are pos * f_i in double.
+//
+// tl_flex_attn_rows serves one query token and HB query heads of one key
+// group per block. Each of the four waves strides over 64-key tiles of the
+// visible range (one key per lane for the score dot products, one value
+// column per lane for P.V), keeps online-softmax statistics per head, and
+// the waves merge through LDS. With score mixing the block evaluates the
+// raw scores of ALL heads for its keys and mixes them into its own HB rows.
+// With few rows over long ranges the keys are also split over blockIdx.z
+// and a merge kernel finishes the rows. It is exact for any query position,
+// so it serves prompt portions and decoding alike; scores, weights and
+// sums are fp32.
+
+#include "common.hpp"
+
+namespace {
+
+constexpr int PAGE = 128;
+static_assert(PAGE % WAVE_SIZE == 0, "a key tile must not straddle pages");
+constexpr int NWAVE = 4;
+constexpr int BLOCK = NWAVE * WAVE_SIZE;
+
+template <typename T> DEVINLINE float ldv(const T* p);
+template <> DEVINLINE float ldv<float>(const float* p) { return *p; }
+template <> DEVINLINE float ldv<bf16>(const bf16* p) { return bf2f(*p); }
+template <typename T> DEVINLINE void stv(T* p, float v);
+template <> DEVINLINE void stv<float>(float* p, float v) { *p = v; }
+template <> DEVINLINE void stv<bf16>(bf16* p, float v) { *p = f2bf(v); }
+
+// ---------------------------------------------------------------- prepare
+template <typename T>
+__global__ __launch_bounds__(BLOCK) void norm_rope_rows_kernel(
+    const T* __restrict__ src, int ld, int col, int n_heads, int head_dim,
+    const float* __restrict__ norm_w, int norm_cols, float eps, int rot_off,
+    int rot_dims, const double* __restrict__ freqs,
+    const int* __restrict__ tok_seq, const int* __restrict__ tok_pos,
+    const int* __restrict__ table, int P, float* __restrict__ out,
+    T* __restrict__ pool) {
+  __shared__ float red[NWAVE];
+  const int t = blockIdx.x;
+  const int N = n_heads * head_dim;
+  const T* row = src + (int64_t)t * ld + col;
+  float rn = 1.f;
+  if (norm_w) {
+    float ss = 0.f;
+    for (int c = threadIdx.x; c < norm_cols; c += BLOCK) {
+      const float v = ldv<T>(row + c);
+      ss += v * v;
+    }
+    const float tot = block_reduce_sum<NWAVE>(ss, red);
+    rn = 1.0f / sqrtf(tot / (float)norm_cols + eps);
+  }
+  const int pos = tok_pos[t];
+  const int half = rot_dims / 2;
+  int64_t prow = 0;
+  if (pool) {
+    const int page = table[(int64_t)tok_seq[t] * P + pos / PAGE];
+    prow = (int64_t)page * n_heads * PAGE + (pos % PAGE);
+  }
+  for (int c = threadIdx.x; c < N; c += BLOCK) {
+    const int hd = c / head_dim, e = c - hd * head_dim;
+    float x = ldv<T>(row + c);
+    if (norm_w && c < norm_cols) x = x * rn * norm_w[c];
+    const int r = e - rot_off;
+    if (r >= 0 && r < rot_dims) {
+      const int i = r < half ? r : r - half;
+      const int cp = r < half ? c + half : c - half;   // the pair's other
+      float y = ldv<T>(row + cp);
+      if (norm_w && cp < norm_cols) y = y * rn * norm_w[cp];
+      const double ang = (double)pos * freqs[i];
+      const float cs = (float)cos(ang), sn = (float)sin(ang);
+      // (u, v) -> (u cos - v sin, v cos + u sin); x is u or v
+      x = r < half ? x * cs - y * sn : x * cs + y * sn;
+    }
+    if (pool)
+      stv<T>(pool + (prow + (int64_t)hd * PAGE) * head_dim + e, x);
+    else
+      out[(int64_t)t * N + c] = x;
+  }
+}
+
+// -------------------------------------------------------------- attention
+// part row (key split z of token t, head h): m, l, acc[V]
+template <typename TK, int HB, int VR, bool TALK>
+__global__ __launch_bounds__(BLOCK) void flex_attn_row_kernel(
+    const float* __restrict__ q, const TK* __restrict__ kpool,
+    const TK* __restrict__ vpool, int vld, const int* __restrict__ tok_seq,
+    const int* __restrict__ tok_pos, const int* __restrict__ table, int P,
+    const float* __restrict__ talk, void* __restrict__ out, int out_f32,
+    float* __restrict__ part, int H, int G, int DK, int V, float scale,
+    int window, int sink) {
+  extern __shared__ float lds[];
+  const int t = blockIdx.x, h0 = blockIdx.y * HB;
+  const int ns = gridDim.z, z = blockIdx.z;
+  const int rep = H / G;
+  const int g0 = h0 / rep;           // key group of this block's heads
+  const int lane = threadIdx.x & (WAVE_SIZE - 1);
+  const int wave = threadIdx.x / WAVE_SIZE;
+  const int NQ = TALK ? H : HB;      // query rows staged
+  const int qbase = TALK ? 0 : h0;
+  // lds: qs[NQ][DK] | tk[HB][H] | stat[NWAVE][HB][2] | acc[NWAVE][HB][V]
+  float* qs = lds;
+  float* tk = qs + NQ * DK;
+  float* stat = tk + (TALK ? HB * H : 0);
+  float* accs = stat + NWAVE * HB * 2;
+
+  const int seq = tok_seq[t], pos = tok_pos[t];
+  const int* tab = table + (int64_t)seq * P;
+  for (int i = threadIdx.x; i < NQ * DK; i += BLOCK)
+    qs[i] = q[(int64_t)t * H * DK + qbase * DK + i] * scale;
+  if (TALK)
+    for (int i = threadIdx.x; i < HB * H; i += BLOCK)
+      tk[i] = talk[(h0 + i / H) * H + (i % H)];
+  __syncthreads();
+
+  float m[HB], l[HB], a[HB][VR];
+#pragma unroll
+  for (int b = 0; b < HB; ++b) {
+    m[b] = -INFINITY;
+    l[b] = 0.f;
+#pragma unroll
+    for (int r = 0; r < VR; ++r) a[b][r] = 0.f;
+  }
+  const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+  const int first = (lo / WAVE_SIZE) * WAVE_SIZE;
+  const bool vec8 = sizeof(TK) == 2 && (DK % 8) == 0;
+  for (int j0 = first + (z * NWAVE + wave) * WAVE_SIZE; j0 <= pos;
+       j0 += ns * NWAVE * WAVE_SIZE) {
+    const int j = j0 + lane;
+    const bool valid = j >= lo && j <= pos;
+    // a 64-key tile lies inside ONE 128-position page
+    const int64_t page_row = (int64_t)tab[j0 / PAGE] * G * PAGE + (j0 % PAGE);
+    float s[HB];
+#pragma unroll
+    for (int b = 0; b < HB; ++b) s[b] = 0.f;
+    if (valid) {
+      if (!TALK) {
+        const TK* kr = kpool + (page_row + (int64_t)g0 * PAGE + lane) * DK;
+        if (vec8) {
+          const bf16x8* k8 = reinterpret_cast<const bf16x8*>(kr);
+          for (int d8 = 0; d8 < DK / 8; ++d8) {
+            const bf16x8 kk = k8[d8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+              const float kd = bf2f(kk.v[e]);
+#pragma unroll
+              for (int b = 0; b < HB; ++b)
+                s[b] += qs[b * DK + d8 * 8 + e] * kd;
+            }
+          }
+        } else {
+          for (int d = 0; d < DK; ++d) {
+            const float kd = ldv<TK>(kr + d);
+#pragma unroll
+            for (int b = 0; b < HB; ++b) s[b] += qs[b * DK + d] * kd;
+          }
+        }
+      } else {
+        for (int hs = 0; hs < H; ++hs) {
+          const TK* kr =
+              kpool + (page_row + (int64_t)(hs / rep) * PAGE + lane) * DK;
+          const float* qh = qs + hs * DK;
+          float raw = 0.f;
+          if (vec8) {
+            const bf16x8* k8 = reinterpret_cast<const bf16x8*>(kr);
+            for (int d8 = 0; d8 < DK / 8; ++d8) {
+              const bf16x8 kk = k8[d8];
+#pragma unroll
+              for (int e = 0; e < 8; ++e)
+                raw += qh[d8 * 8 + e] * bf2f(kk.v[e]);
+            }
+          } else {
+            for (int d = 0; d < DK; ++d) raw += qh[d] * ldv<TK>(kr + d);
+          }
+#pragma unroll
+          for (int b = 0; b < HB; ++b) s[b] += tk[b * H + hs] * raw;
+        }
+      }
+    }
+    float p[HB];
+#pragma unroll
+    for (int b = 0; b < HB; ++b) {
+      const float sv = valid ? s[b] : -INFINITY;
+      const float nm = fmaxf(m[b], wave_reduce_max(sv));
+      // nm is finite: every tile of the loop holds at least one valid key
+      const float c = expf(m[b] - nm);
+      p[b] = valid ? expf(sv - nm) : 0.f;
+      l[b] = l[b] * c + wave_reduce_sum(p[b]);
+      m[b] = nm;
+#pragma unroll
+      for (int r = 0; r < VR; ++r) a[b][r] *= c;
+    }
+    const int jb = max(0, lo - j0), je = min(WAVE_SIZE, pos + 1 - j0);
+    const TK* vtile = vpool + (page_row + (int64_t)g0 * PAGE) * vld;
+    for (int jj = jb; jj < je; ++jj) {
+      float w[HB];
+#pragma unroll
+      for (int b = 0; b < HB; ++b) w[b] = __shfl(p[b], jj, WAVE_SIZE);
+      const TK* vr = vtile + (int64_t)jj * vld;
+#pragma unroll
+      for (int r = 0; r < VR; ++r) {
+        const int c = lane + r * WAVE_SIZE;
+        if (c < V) {
+          const float vv = ldv<TK>(vr + c);
+#pragma unroll
+          for (int b = 0; b < HB; ++b) a[b][r] += w[b] * vv;
+        }
+      }
+    }
+  }
+  // a wave whose tiles were all beyond the range keeps m = -inf, l = 0
+#pragma unroll
+  for (int b = 0; b < HB; ++b) {
+    if (lane == 0) {
+      stat[(wave * HB + b) * 2 + 0] = m[b];
+      stat[(wave * HB + b) * 2 + 1] = l[b];
+    }
+#pragma unroll
+    for (int r = 0; r < VR; ++r) {
+      const int c = lane + r * WAVE_SIZE;
+      if (c < V) accs[(wave * HB + b) * V + c] = a[b][r];
+    }
+  }
+  __syncthreads();
+  for (int b = 0; b < HB; ++b) {
+    float M = -INFINITY;
+    for (int w = 0; w < NWAVE; ++w) M = fmaxf(M, stat[(w * HB + b) * 2]);
+    float f[NWAVE], L = 0.f;
+    if (ns > 1) {
+      // partial of this key split; an empty split stores m = -inf, l = 0
+      for (int w = 0; w < NWAVE; ++w) {
+        const float mw = stat[(w * HB + b) * 2];
+        f[w] = (mw == -INFINITY) ? 0.f : expf(mw - M);
+        L += f[w] * stat[(w * HB + b) * 2 + 1];
+      }
+      float* pr = part + (((int64_t)t * H + h0 + b) * ns + z) * (2 + V);
+      if (threadIdx.x == 0) {
+        pr[0] = M;
+        pr[1] = L;
+      }
+      for (int c = threadIdx.x; c < V; c += BLOCK) {
+        float A = 0.f;
+        for (int w = 0; w < NWAVE; ++w) A += f[w] * accs[(w * HB + b) * V + c];
+        pr[2 + c] = A;
+      }
+      continue;
+    }
+    if (sink) M = fmaxf(M, 0.f);
+    for (int w = 0; w < NWAVE; ++w) {
+      const float mw = stat[(w * HB + b) * 2];
+      f[w] = (mw == -INFINITY) ? 0.f : expf(mw - M);
+      L += f[w] * stat[(w * HB + b) * 2 + 1];
+    }
+    if (sink) L += expf(-M);
+    for (int c = threadIdx.x; c < V; c += BLOCK) {
+      float A = 0.f;
+      for (int w = 0; w < NWAVE; ++w) A += f[w] * accs[(w * HB + b) * V + c];
+      const int64_t o = ((int64_t)t * H + h0 + b) * V + c;
+      if (out_f32)
+        ((float*)out)[o] = A / L;
+      else
+        ((bf16*)out)[o] = f2bf(A / L);
+    }
+  }
+}
+
+// one block per (token, head): merge the key splits
+__global__ __launch_bounds__(BLOCK) void flex_attn_merge_kernel(
+    const float* __restrict__ part, void* __restrict__ out, int out_f32,
+    int ns, int V, int sink) {
+  const int64_t row = blockIdx.x;
+  const float* pr = part + row * ns * (2 + V);
+  float M = -INFINITY;
+  for (int z = 0; z < ns; ++z) M = fmaxf(M, pr[z * (2 + V)]);
+  if (sink) M = fmaxf(M, 0.f);
+  float L = sink ? expf(-M) : 0.f;
+  for (int z = 0; z < ns; ++z) {
+    const float mz = pr[z * (2 + V)];
+    L += (mz == -INFINITY ? 0.f : expf(mz - M)) * pr[z * (2 + V) + 1];
+  }
+  for (int c = threadIdx.x; c < V; c += BLOCK) {
+    float A = 0.f;
+    for (int z = 0; z < ns; ++z) {
+      const float mz = pr[z * (2 + V)];
+      A += (mz == -INFINITY ? 0.f : expf(mz - M)) * pr[z * (2 + V) + 2 + c];
+    }
+    if (out_f32)
+      ((float*)out)[row * V + c] = A / L;
+    else
+      ((bf16*)out)[row * V + c] = f2bf(A / L);
+  }
+}
+
+template <typename TK, int HB, int VR>
+void launch_rows(bool has_talk, dim3 grid, size_t smem, hipStream_t stream,
+                 const float* q, const TK* kpool, const TK* vpool, int vld,
+                 const int* tok_seq, const int* tok_pos, const int* table,
+                 int P, const float* talk, void* out, int out_f32,
+                 float* part, int H, int G, int DK, int V, float scale,
+                 int window, int sink) {
+  if (has_talk)
+    hipLaunchKernelGGL((flex_attn_row_kernel<TK, HB, VR, true>), grid,
+                       dim3(BLOCK), smem, stream, q, kpool, vpool, vld,
+                       tok_seq, tok_pos, table, P, talk, out, out_f32, part,
+                       H, G, DK, V, scale, window, sink);
+  else
+    hipLaunchKernelGGL((flex_attn_row_kernel<TK, HB, VR, false>), grid,
+                       dim3(BLOCK), smem, stream, q, kpool, vpool, vld,
+                       tok_seq, tok_pos, table, P, talk, out, out_f32, part,
+                       H, G, DK, V, scale, window, sink);
+}
+
+size_t rows_smem(bool has_talk, int hb, int H, int DK, int V) {
+  return sizeof(float) * ((size_t)(has_talk ? H : hb) * DK +
+                          (has_talk ? (size_t)hb * H : 0) +
+                          (size_t)NWAVE * hb * 2 + (size_t)NWAVE * hb * V);
+}
+
+}  // namespace
+
+extern "C" {
+
+void tl_norm_rope_rows(const void* src, int ld, int col, int n_heads,
+                       int head_dim, const void* norm_w, int norm_cols,
+                       float eps, int rot_off, int rot_dims,
+                       const void* freqs, const void* tok_seq,
+                       const void* tok_pos, const void* table, int P, int T,
+                       void* out, void* pool, int is_f32,
+                       hipStream_t stream) {
+  if (T <= 0) return;
+  dim3 grid(T), block(BLOCK);
+  if (is_f32)
+    hipLaunchKernelGGL(norm_rope_rows_kernel<float>, grid, block, 0, stream,
+                       (const float*)src, ld, col, n_heads, head_dim,
+                       (const float*)norm_w, norm_cols, eps, rot_off,
+                       rot_dims, (const double*)freqs, (const int*)tok_seq,
+                       (const int*)tok_pos, (const int*)table, P,
+                       (float*)out, (float*)pool);
+  else
+    hipLaunchKernelGGL(norm_rope_rows_kernel<bf16>, grid, block, 0, stream,
+                       (const bf16*)src, ld, col, n_heads, head_dim,
+                       (const float*)norm_w, norm_cols, eps, rot_off,
+                       rot_dims, (const double*)freqs, (const int*)tok_seq,
+                       (const int*)tok_pos, (const int*)table, P,
+                       (float*)out, (bf16*)pool);
+}
+
+// heads per block for a shape: the largest of 8, 4, 2, 1 that divides the
+// heads per key group and fits the register and LDS budgets; 0 if none
+int tl_flex_attn_heads_per_block(int H, int G, int DK, int V, int has_talk) {
+  if (V > 512 || G <= 0 || H % G != 0) return 0;
+  const int vr = (V + WAVE_SIZE - 1) / WAVE_SIZE;
+  const int vrr = vr <= 1 ? 1 : vr <= 2 ? 2 : vr <= 4 ? 4 : 8;
+  for (int hb = 8; hb >= 1; hb >>= 1) {
+    if ((H / G) % hb != 0 || hb * vrr > 32) continue;
+    if (rows_smem(has_talk != 0, hb, H, DK, V) <= 64 * 1024) return hb;
+  }
+  return 0;
+}
+
+// returns 0 on success, 1 if the shape is outside what the kernel serves
+int tl_flex_attn_rows(const void* q, const void* kpool, const void* vpool,
+                      int vld, const void* tok_seq, const void* tok_pos,
+                      const void* table, int P, const void* talk, void* out,
+                      int out_f32, void* part, int ns, int T, int H, int G,
+                      int DK, int V, float scale, int window, int sink,
+                      int pool_f32, hipStream_t stream) {
+  if (T <= 0) return 0;
+  const bool has_talk = talk != nullptr;
+  const int hb = tl_flex_attn_heads_per_block(H, G, DK, V, has_talk ? 1 : 0);
+  if (hb == 0 || ns < 1 || (ns > 1 && !part)) return 1;
+  const int vr = (V + WAVE_SIZE - 1) / WAVE_SIZE;
+  const size_t smem = rows_smem(has_talk, hb, H, DK, V);
+  dim3 grid(T, H / hb, ns);
+#define TL_FA(TT, HBB, VRR)                                                  \
+  launch_rows<TT, HBB, VRR>(has_talk, grid, smem, stream, (const float*)q,   \
+                            (const TT*)kpool, (const TT*)vpool, vld,         \
+                            (const int*)tok_seq, (const int*)tok_pos,        \
+                            (const int*)table, P, (const float*)talk, out,   \
+                            out_f32, (float*)part, H, G, DK, V, scale,       \
+                            window, sink)
+#define TL_FA_V(TT, HBB)                     \
+  if (vr <= 1) TL_FA(TT, HBB, 1);            \
+  else if (vr <= 2) TL_FA(TT, HBB, 2);       \
+  else if (vr <= 4) TL_FA(TT, HBB, 4);       \
+  else if (HBB <= 4) TL_FA(TT, (HBB <= 4 ? HBB : 4), 8);
+#define TL_FA_H(TT)                    \
+  if (hb == 8) { TL_FA_V(TT, 8) }      \
+  else if (hb == 4) { TL_FA_V(TT, 4) } \
+  else if (hb == 2) { TL_FA_V(TT, 2) } \
+  else { TL_FA_V(TT, 1) }
+  if (pool_f32) {
+    TL_FA_H(float)
+  } else {
+    TL_FA_H(bf16)
+  }
+#undef TL_FA_H
+#undef TL_FA_V
+#undef TL_FA
+  if (ns > 1)
+    hipLaunchKernelGGL(flex_attn_merge_kernel, dim3(T * H), dim3(BLOCK), 0,
+                       stream, (const float*)part, out, out_f32, ns, V, sink);
+  return 0;
+}
+
+}  // extern "C"

@@ -493,10 +493,19 @@ def flex_attention(q: torch.Tensor, kpool: torch.Tensor,
     T = q.shape[0]
     assert q.dtype == torch.float32 and q.shape[1] == H * DK
     if q.is_cuda:
+        # few rows over long key ranges (decoding): spread each row's
+        # keys over several blocks so the chip is filled; a function of
+        # the step's shape only
+        span = min(meta.max_kv, window) if window > 0 else meta.max_kv
+        n_split = 1
+        while (n_split < 16 and meta.T * H * n_split < 1024
+               and span > 512 * n_split):
+            n_split *= 2
         return _ext().flex_attn_rows(q, kpool, vpool, meta.tok_seq,
                                      meta.tok_pos, meta.table, talk, int(H),
                                      float(scale), int(window), bool(sink),
-                                     int(V), out_dtype == torch.float32)
+                                     int(V), out_dtype == torch.float32,
+                                     n_split)
     out = torch.empty(T, H, V)
     qf = q.view(T, H, DK)
     rep = H // G
