@@ -274,9 +274,10 @@ class LightningMixer(nn.Module, _F32Cache):
         self.proj = TLLinear(width, 2 * hd + 2 * hv, bias=False)
         self.norm = nn.Parameter(torch.ones(hv))
         self.o_proj = TLLinear(hv, width, bias=False)
-        self.register_buffer("decay", torch.tensor(
-            [float(x) for x in decay], dtype=torch.float64),
-            persistent=False)
+        # a constant of the design, not a parameter: kept out of the
+        # module's tensors so that a cast of the module to the serving
+        # dtype cannot round it
+        self.decay = tuple(float(x) for x in decay)
 
     def cache_spec(self):
         return {"kind": "state", "shapes": [(self.H, self.D, self.V)]}
@@ -284,7 +285,8 @@ class LightningMixer(nn.Module, _F32Cache):
     def _decay32(self, dev):
         hit = self.__dict__.get("_dec")
         if hit is None or hit.device != dev:
-            hit = self.decay.to(device=dev, dtype=torch.float32)
+            hit = torch.tensor(self.decay, dtype=torch.float64).to(
+                device=dev, dtype=torch.float32)
             self.__dict__["_dec"] = hit
         return hit
 
