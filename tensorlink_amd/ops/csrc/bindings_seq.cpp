@@ -33,6 +33,14 @@ int tl_flex_attn_rows(const void* q, const void* kpool, const void* vpool,
                       int out_f32, void* part, int ns, int T, int H, int G,
                       int DK, int V, float scale, int window, int sink,
                       int pool_f32, hipStream_t stream);
+int tl_flex_attn_tiles_ok(int H, int G, int KG, int DK, int V);
+void tl_stage_queries(const void* q, const void* talk, void* out, int T,
+                      int H, int G, int DK, hipStream_t stream);
+int tl_flex_attn_tiles(const void* q, const void* kpool, const void* vpool,
+                       int vld, const void* tiles, int n_tiles,
+                       const void* table, int P, void* out, int out_f32,
+                       int H, int G, int KG, int DK, int V, float scale,
+                       int window, int sink, hipStream_t stream);
 int tl_lightning_scan(const void* proj, int ld, int q_off, int k_off,
                       int v_off, const void* decay, void* S, const void* cu,
                       const void* slots, const void* pos0, void* out, int B,
@@ -259,6 +267,70 @@ Tensor flex_attn_rows(Tensor q, Tensor kpool, c10::optional<Tensor> vpool,
   return out;
 }
 
+bool flex_attn_tiles_ok(int64_t H, int64_t G, bool has_talk, int64_t DK,
+                        int64_t V) {
+  return tl_flex_attn_tiles_ok((int)H, (int)G, has_talk ? (int)G : 1,
+                               (int)DK, (int)V) != 0;
+}
+
+// MFMA path for prompt portions (bf16 pools): `tiles` [n, 4] int32 rows of
+// (sequence, first flat token, token count <= 64, first position).
+Tensor flex_attn_tiles(Tensor q, Tensor kpool, c10::optional<Tensor> vpool,
+                       Tensor tiles, Tensor table,
+                       c10::optional<Tensor> talk, int64_t H, double scale,
+                       int64_t window, bool sink, int64_t V, bool out_f32) {
+  SEQ_F32(q);
+  SEQ_IN(kpool);
+  SEQ_I32(tiles);
+  SEQ_I32(table);
+  TORCH_CHECK(kpool.scalar_type() == torch::kBFloat16 && kpool.dim() == 4 &&
+                  kpool.size(2) == 128,
+              "key pool must be bf16 [pages, G, 128, DK]");
+  const int G = kpool.size(1), DK = kpool.size(3);
+  const int64_t T = q.size(0);
+  TORCH_CHECK(q.dim() == 2 && q.size(1) == H * DK, "q must be [T, H*DK]");
+  TORCH_CHECK(tiles.dim() == 2 && tiles.size(1) == 4 && table.dim() == 2,
+              "tiles must be [n, 4]");
+  const void* vp = kpool.data_ptr();
+  int vld = DK;
+  if (vpool.has_value()) {
+    SEQ_IN(vpool.value());
+    TORCH_CHECK(vpool->scalar_type() == torch::kBFloat16 &&
+                    vpool->dim() == 4 && vpool->size(0) == kpool.size(0) &&
+                    vpool->size(1) == G && vpool->size(2) == 128 &&
+                    vpool->size(3) == V,
+                "value pool must be bf16 [pages, G, 128, V]");
+    vp = vpool->data_ptr();
+    vld = V;
+  } else {
+    TORCH_CHECK(G == 1 && V >= 1 && V <= DK,
+                "values are a prefix of the single key head's row");
+  }
+  if (talk.has_value()) {
+    SEQ_F32(talk.value());
+    TORCH_CHECK(talk->numel() == H * H, "talk must be [H, H]");
+  }
+  const int KG = talk.has_value() ? G : 1;
+  TORCH_CHECK(tl_flex_attn_tiles_ok((int)H, G, KG, DK, (int)V),
+              "flex_attn_tiles: shape outside the kernel's range");
+  auto qs = torch::empty({T, H * KG * DK},
+                         q.options().dtype(torch::kBFloat16));
+  auto out = torch::empty(
+      {T, H * V}, q.options().dtype(out_f32 ? torch::kFloat
+                                            : torch::kBFloat16));
+  if (T == 0 || tiles.size(0) == 0) return out;
+  tl_stage_queries(q.data_ptr(),
+                   talk.has_value() ? talk->data_ptr() : nullptr,
+                   qs.data_ptr(), (int)T, (int)H, G, DK, seq_stream());
+  const int rc = tl_flex_attn_tiles(
+      qs.data_ptr(), kpool.data_ptr(), vp, vld, tiles.data_ptr(),
+      (int)tiles.size(0), table.data_ptr(), (int)table.size(1),
+      out.data_ptr(), out_f32 ? 1 : 0, (int)H, G, KG, DK, (int)V,
+      (float)scale, (int)window, sink ? 1 : 0, seq_stream());
+  TORCH_CHECK(rc == 0, "flex_attn_tiles: launch refused");
+  return out;
+}
+
 Tensor lightning_scan(Tensor proj, int64_t q_off, int64_t k_off,
                       int64_t v_off, Tensor decay, Tensor S, Tensor cu,
                       Tensor slots, Tensor pos0, int64_t H, int64_t D,
@@ -306,6 +378,10 @@ void register_seq_ops(pybind11::module& mod) {
           "scattered into a page pool");
   mod.def("flex_attn_rows", &flex_attn_rows,
           "paged softmax attention: window, sink, score mixing, latent rows");
+  mod.def("flex_attn_tiles_ok", &flex_attn_tiles_ok,
+          "whether the MFMA tile kernel serves a shape");
+  mod.def("flex_attn_tiles", &flex_attn_tiles,
+          "paged softmax attention on MFMA, 64-query tiles (bf16 pools)");
   mod.def("lightning_scan", &lightning_scan,
           "decayed linear attention over ragged sequences (slot state)");
 }

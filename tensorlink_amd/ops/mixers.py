@@ -493,6 +493,15 @@ def flex_attention(q: torch.Tensor, kpool: torch.Tensor,
     T = q.shape[0]
     assert q.dtype == torch.float32 and q.shape[1] == H * DK
     if q.is_cuda:
+        if (kpool.dtype == torch.bfloat16 and meta.T > meta.B
+                and not os.environ.get("TL_NO_ATTN_TILES")
+                and _ext().flex_attn_tiles_ok(H, G, talk is not None, DK,
+                                              V)):
+            # a prompt portion is in the step: 64-query MFMA tiles
+            return _ext().flex_attn_tiles(
+                q, kpool, vpool, meta.query_tiles(), meta.table, talk,
+                int(H), float(scale), int(window), bool(sink), int(V),
+                out_dtype == torch.float32)
         # few rows over long key ranges (decoding): spread each row's
         # keys over several blocks so the chip is filled; a function of
         # the step's shape only

@@ -103,6 +103,24 @@ def cfg_wide():
                  "mixer": lit(2, 40, 136, [0.9, 0.99]), "mlp": None}]}
 
 
+def cfg_tiles():
+    """Head sizes the MFMA prompt kernel serves in bf16 (key size a
+    multiple of 8, value size of 16): mixed scores over two key heads, a
+    window that is no multiple of the key tile, latents shared."""
+    return {"architecture": "Senulix", "vocab": 70, "width": 64,
+            "norm": {"eps": 1e-6}, "token_side": {"dim": 8},
+            "logit_softcap": 20.0, "layers": [
+                {"type": "latent_attention", "mixer": lat(4, 16, 8, 32, 48),
+                 "mlp": {"kind": "dense", "ff": 128}},
+                {"type": "attention", "mixer": att(4, 2, 24, 48, 8, 70),
+                 "mlp": None},
+                {"type": "lightning",
+                 "mixer": lit(2, 32, 64, [0.96, 0.995]), "mlp": None},
+                {"type": "latent_attention",
+                 "mixer": lat(2, 24, 8, 16, 48, kv_from=0),
+                 "mlp": {"kind": "dense", "ff": 128}}]}
+
+
 def mixer_weights(lc, w, rnd):
     """Checkpoint tensors of one mixer (names without the layer prefix)."""
     mc, P = lc["mixer"], {}
@@ -483,6 +501,52 @@ def test_window_edges_and_sink(device, dtype):
                 assert mixer_close(got, want, dtype), (qpos, dist, cuts)
 
 
+@pytest.mark.gpu
+def test_tile_kernel_against_row_kernel_and_plain():
+    """bf16 pools on the GPU: a step with a prompt portion takes the MFMA
+    tile kernel, a step of single tokens the row kernel; both against the
+    plain torch form, over windows below, at and above the key tile, sink
+    on and off, mixed scores over several key heads, values inside the
+    key row, ragged portions beside single tokens."""
+    g = torch.Generator().manual_seed(11)
+    dev, dt = "cuda", torch.bfloat16
+    new, pos0, slots = [70, 1, 200, 3], [0, 130, 60, 300], [2, 0, 1, 3]
+    table = torch.tensor([[3, 1, 0, 0], [4, 5, 2, 0], [6, 7, 8, 0],
+                          [9, 10, 11, 0]], dtype=torch.int32)
+    mc = mx.RaggedMeta(new, pos0, slots, table, "cpu")
+    mg = mx.RaggedMeta(new, pos0, slots, table.to(dev), dev)
+    # the same tokens one by one: every row alone in its step
+    T = sum(new)
+    for H, G, D, V, win, sink, talk in (
+            (4, 2, 24, 48, 37, True, True), (6, 1, 56, 0, 0, False, False),
+            (8, 2, 64, 64, 64, True, False), (3, 3, 16, 128, 7, False, True),
+            (8, 4, 32, 32, 150, True, True), (2, 1, 40, 32, 1, True, False)):
+        kp = torch.randn(12, G, 128, D, generator=g).to(dt)
+        vp = torch.randn(12, G, 128, V, generator=g).to(dt) if V else None
+        q = torch.randn(T, H * D, generator=g)
+        tk = (torch.eye(H) + 0.3 * torch.randn(H, H, generator=g)) \
+            if talk else None
+        kw = dict(window=win, sink=sink, v_cols=0 if V else 48)
+        want = mx.flex_attention(q, kp, vp, mc, H, 0.15, talk=tk, **kw)
+        assert mx._ext().flex_attn_tiles_ok(H, G, talk, D, V or 48)
+        got = mx.flex_attention(
+            q.to(dev), kp.to(dev), vp.to(dev) if V else None, mg, H, 0.15,
+            talk=tk.to(dev) if talk else None, **kw)
+        assert (got.cpu() - want).abs().max() < 2e-2 * want.abs().max()
+        rows = []
+        for t in range(T):
+            b = int(mc.tok_seq[t])
+            m1 = mx.RaggedMeta([1], [int(mc.tok_pos[t])], [slots[b]],
+                               table[[b]].to(dev), dev)
+            rows.append(mx.flex_attention(
+                q[t:t + 1].to(dev), kp.to(dev), vp.to(dev) if V else None,
+                m1, H, 0.15, talk=tk.to(dev) if talk else None, **kw))
+            if t > 80 and t % 7:
+                rows[-1] = got[t:t + 1]          # a sample of rows is enough
+        assert (torch.cat(rows).cpu() - want).abs().max() < \
+            2e-2 * want.abs().max()
+
+
 @pytest.mark.parametrize("device,dtype", ALL)
 def test_rowwise_ops(device, dtype):
     """Post-norm residual (both weight forms), gated scaling, both GELUs
@@ -526,8 +590,8 @@ def test_rowwise_ops(device, dtype):
 
 
 # ---------------------------------------------------------- whole model
-@pytest.mark.parametrize("cfg_fn", [cfg_mixed, cfg_ones, cfg_wide],
-                         ids=lambda f: f.__name__)
+@pytest.mark.parametrize("cfg_fn", [cfg_mixed, cfg_ones, cfg_wide,
+                                    cfg_tiles], ids=lambda f: f.__name__)
 @pytest.mark.parametrize("device,dtype", ALL)
 def test_whole_prompt_and_layers(tmp_path_factory, device, dtype, cfg_fn):
     """Logits of a whole prompt and the residual after every layer."""
@@ -553,8 +617,8 @@ def test_whole_prompt_and_layers(tmp_path_factory, device, dtype, cfg_fn):
             assert float(err.max()) < 0.5, li
 
 
-@pytest.mark.parametrize("cfg_fn", [cfg_mixed, cfg_ones, cfg_wide],
-                         ids=lambda f: f.__name__)
+@pytest.mark.parametrize("cfg_fn", [cfg_mixed, cfg_ones, cfg_wide,
+                                    cfg_tiles], ids=lambda f: f.__name__)
 @pytest.mark.parametrize("device,dtype", ALL)
 def test_portions_and_decoding(tmp_path_factory, device, dtype, cfg_fn):
     """Prefill against token-by-token decoding from the first token, and
