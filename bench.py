@@ -49,6 +49,10 @@ def parse_args():
                         "beside an equal-size Qwen3-MoE-shaped model")
     p.add_argument("--sizes", default="w1024,w2048",
                    help="layered mode: comma list of size presets")
+    p.add_argument("--family", choices=["kepusun", "senulix"],
+                   default="kepusun",
+                   help="layered mode: which layered family to time "
+                        "(senulix: beside an equal-size dense GQA decoder)")
     p.add_argument("--dp", type=int, default=1,
                    help="data-parallel replicas (train mode; world=dp*pp)")
     return p.parse_args()
@@ -146,6 +150,59 @@ def layered_configs(z):
     return kep, ref
 
 
+SENULIX_SIZES = {
+    # layers: latent, windowed, windowed, lightning, latent (shared), windowed
+    "w1024": dict(width=1024, heads=8, kv=2, dim=128, rot=64, rank=192,
+                  window=1024, ff=4096, side=32, vocab=32000, batch=8,
+                  prompt=2048),
+    "w2048": dict(width=2048, heads=16, kv=4, dim=128, rot=64, rank=192,
+                  window=1024, ff=8192, side=64, vocab=32000, batch=8,
+                  prompt=2048),
+    "tiny": dict(width=128, heads=2, kv=1, dim=32, rot=16, rank=48,
+                 window=64, ff=256, side=8, vocab=512, batch=2, prompt=96),
+}
+
+
+def senulix_configs(z):
+    """(Senulix config, equal-size dense GQA decoder) of a preset: same
+    width, depth, vocabulary, head count and head size; the gated
+    three-matrix feed-forward of the dense model gets 2/3 of the
+    two-matrix one's width, which equalises their parameters."""
+    from tensorlink_amd.models.configs import ModelConfig
+    from tensorlink_amd.models.senulix import SenulixConfig
+    H, D = z["heads"], z["dim"]
+    mlp = {"kind": "dense", "ff": z["ff"]}
+    la = {"heads": H, "dim": D, "rot_dim": z["rot"], "vdim": D,
+          "kv_rank": z["rank"], "scale": (D + z["rot"]) ** -0.5,
+          "rot": {"dims": z["rot"], "base": 10000.0}}
+    wa = {"heads": H, "kv_heads": z["kv"], "dim": D, "vdim": D,
+          "scale": D ** -0.5, "rot": {"dims": z["rot"], "base": 50000.0},
+          "mask": {"size": z["window"]}}
+    li = {"heads": H, "dim": D, "vdim": D,
+          "decay": [1.0 - 2.0 ** (-3 - 5 * i / max(1, H - 1))
+                    for i in range(H)]}
+    layers = [{"type": "latent_attention", "mixer": la, "mlp": mlp},
+              {"type": "attention", "mixer": wa, "mlp": mlp},
+              {"type": "attention", "mixer": wa, "mlp": mlp},
+              {"type": "lightning", "mixer": li, "mlp": None},
+              {"type": "latent_attention", "mixer": dict(la, kv_from=0),
+               "mlp": mlp},
+              {"type": "attention", "mixer": wa, "mlp": mlp}]
+    sen = SenulixConfig.from_dict({
+        "architecture": "Senulix", "vocab": z["vocab"], "width": z["width"],
+        "norm": {"eps": 1e-6}, "token_side": {"dim": z["side"]},
+        "logit_softcap": 30.0, "layers": layers},
+        name="senulix-" + str(z["width"]))
+    ref = ModelConfig(
+        name="dense-gqa-" + str(z["width"]), vocab_size=z["vocab"],
+        hidden_size=z["width"],
+        intermediate_size=(2 * z["ff"] // 3 + 63) // 64 * 64,
+        num_hidden_layers=len(layers), num_attention_heads=H,
+        num_key_value_heads=z["kv"], head_dim=D,
+        max_position_embeddings=8192, architecture="qwen3")
+    return sen, ref
+
+
 @torch.no_grad()
 def run_layered(args, device, use_gpu):
     """Prefill and decode tokens/s of the Kepusun family beside the
@@ -195,10 +252,18 @@ def run_layered(args, device, use_gpu):
         return out
 
     for name in args.sizes.split(","):
-        z = LAYERED_SIZES[name]
-        kep, ref = layered_configs(z)
-        B, S = z["batch"], z["prompt"]
-        res = {"kepusun": measure(kep, B, S), "qwen3_moe": measure(ref, B, S)}
+        if args.family == "senulix":
+            z = SENULIX_SIZES[name]
+            sen, ref = senulix_configs(z)
+            B, S = z["batch"], z["prompt"]
+            res = {"senulix": measure(sen, B, S),
+                   "dense_gqa": measure(ref, B, S)}
+        else:
+            z = LAYERED_SIZES[name]
+            kep, ref = layered_configs(z)
+            B, S = z["batch"], z["prompt"]
+            res = {"kepusun": measure(kep, B, S),
+                   "qwen3_moe": measure(ref, B, S)}
         print(json.dumps({
             "metric": "layered-family prefill/decode tokens/sec",
             "size": name, "batch": B, "prompt_len": S, "new_tokens": new,
