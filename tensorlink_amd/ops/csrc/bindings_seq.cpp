@@ -45,6 +45,17 @@ int tl_lightning_scan(const void* proj, int ld, int q_off, int k_off,
                       int v_off, const void* decay, void* S, const void* cu,
                       const void* slots, const void* pos0, void* out, int B,
                       int H, int D, int V, int is_f32, hipStream_t stream);
+void tl_lightning_chunk_prep(const void* proj, int ld, int q_off, int k_off,
+                             int v_off, const void* decay, const void* cu_c,
+                             void* Qs, void* Qd, void* Ks, void* Kw, void* Vs,
+                             int NC, int H, int D, int V, int C, int is_f32,
+                             hipStream_t stream);
+void tl_lightning_decay_mask(void* A, const void* decay, int NCH, int H,
+                             int C, hipStream_t stream);
+void tl_lightning_chain(void* U, void* S, const void* decay, const void* cu_c,
+                        const void* chunk_base, const void* n_chunks,
+                        const void* slots, const void* pos0, int B, int H,
+                        int DV, hipStream_t stream);
 }
 
 namespace {
@@ -364,9 +375,79 @@ Tensor lightning_scan(Tensor proj, int64_t q_off, int64_t k_off,
   return out;
 }
 
+// silu(q), a^(i+1) silu(q), silu(k), a^(n-1-j) silu(k), silu(v) per
+// (chunk, head), zero-padded to C rows: five fp32 tensors [NC*H, C, D|V]
+std::vector<Tensor> lightning_chunk_prep(Tensor proj, int64_t q_off,
+                                         int64_t k_off, int64_t v_off,
+                                         Tensor decay, Tensor cu_c,
+                                         int64_t H, int64_t D, int64_t V,
+                                         int64_t C) {
+  SEQ_IN(proj);
+  SEQ_F32(decay);
+  SEQ_I32(cu_c);
+  TORCH_CHECK(proj.dim() == 2 && cu_c.numel() >= 1, "proj [T, L], cu_c");
+  const int64_t ld = proj.size(1), NC = cu_c.numel() - 1;
+  TORCH_CHECK(q_off + H * D <= ld && k_off + H * D <= ld &&
+                  v_off + H * V <= ld && decay.numel() == H && C >= 1,
+              "projection columns out of range");
+  auto o = proj.options().dtype(torch::kFloat);
+  std::vector<Tensor> r;
+  for (int i = 0; i < 4; ++i) r.push_back(torch::empty({NC * H, C, D}, o));
+  r.push_back(torch::empty({NC * H, C, V}, o));
+  tl_lightning_chunk_prep(proj.data_ptr(), (int)ld, (int)q_off, (int)k_off,
+                          (int)v_off, decay.data_ptr(), cu_c.data_ptr(),
+                          r[0].data_ptr(), r[1].data_ptr(), r[2].data_ptr(),
+                          r[3].data_ptr(), r[4].data_ptr(), (int)NC, (int)H,
+                          (int)D, (int)V, (int)C, act_is_f32(proj),
+                          seq_stream());
+  return r;
+}
+
+void lightning_decay_mask_(Tensor A, Tensor decay) {
+  SEQ_F32(A);
+  SEQ_F32(decay);
+  const int H = decay.numel();
+  TORCH_CHECK(A.dim() == 3 && A.size(1) == A.size(2) && A.size(0) % H == 0,
+              "A must be [chunks*H, C, C]");
+  tl_lightning_decay_mask(A.data_ptr(), decay.data_ptr(), (int)A.size(0), H,
+                          (int)A.size(1), seq_stream());
+}
+
+void lightning_chain_(Tensor U, Tensor S, Tensor decay, Tensor cu_c,
+                      Tensor chunk_base, Tensor n_chunks, Tensor slots,
+                      Tensor pos0) {
+  SEQ_F32(U);
+  SEQ_F32(S);
+  SEQ_F32(decay);
+  SEQ_I32(cu_c);
+  SEQ_I32(chunk_base);
+  SEQ_I32(n_chunks);
+  SEQ_I32(slots);
+  SEQ_I32(pos0);
+  const int H = decay.numel();
+  TORCH_CHECK(S.dim() == 4 && S.size(1) == H, "S pool [slots, H, D, V]");
+  const int64_t DV = S.size(2) * S.size(3);
+  const int64_t NC = cu_c.numel() - 1;
+  TORCH_CHECK(U.numel() == NC * H * DV, "U must be [chunks*H, D, V]");
+  const int B = slots.size(0);
+  TORCH_CHECK(chunk_base.size(0) == B && n_chunks.size(0) == B &&
+                  pos0.size(0) == B,
+              "per-sequence chunk metadata");
+  tl_lightning_chain(U.data_ptr(), S.data_ptr(), decay.data_ptr(),
+                     cu_c.data_ptr(), chunk_base.data_ptr(),
+                     n_chunks.data_ptr(), slots.data_ptr(), pos0.data_ptr(),
+                     B, H, (int)DV, seq_stream());
+}
+
 }  // namespace
 
 void register_seq_ops(pybind11::module& mod) {
+  mod.def("lightning_chunk_prep", &lightning_chunk_prep,
+          "per-chunk activations of the chunk form of lightning attention");
+  mod.def("lightning_decay_mask_", &lightning_decay_mask_,
+          "A[i][j] *= a^(i-j) below and on the diagonal, 0 above");
+  mod.def("lightning_chain_", &lightning_chain_,
+          "chunk summaries -> state before each chunk; final state to slot");
   mod.def("postnorm_add", &postnorm_add,
           "X += y / rms(y) * g on the fp32 residual; returns the cast copy");
   mod.def("rms_scale", &rms_scale, "x / rms(x) * g [* sigmoid(gate)]");

@@ -14,8 +14,11 @@
 // group per block. Each of the four waves strides over 64-key tiles of the
 // visible range (one key per lane for the score dot products, one value
 // column per lane for P.V), keeps online-softmax statistics per head, and
-// the waves merge through LDS. With score mixing the block evaluates the
-// raw scores of ALL heads for its keys and mixes them into its own HB rows.
+// the waves merge through LDS. Score mixing is linear and heads of one key
+// group share their key, so the mixed score of head h is one dot product
+// between the mixed query [sum_{g in c} T[h,g] q_g]_c and the G key heads'
+// rows side by side: the block stages mixed queries and then works as if
+// the key were G times as wide.
 // With few rows over long ranges the keys are also split over blockIdx.z
 // and a merge kernel finishes the rows. It is exact for any query position,
 // so it serves prompt portions and decoding alike; scores, weights and
@@ -106,21 +109,28 @@ __global__ __launch_bounds__(BLOCK) void flex_attn_row_kernel(
   const int g0 = h0 / rep;           // key group of this block's heads
   const int lane = threadIdx.x & (WAVE_SIZE - 1);
   const int wave = threadIdx.x / WAVE_SIZE;
-  const int NQ = TALK ? H : HB;      // query rows staged
-  const int qbase = TALK ? 0 : h0;
-  // lds: qs[NQ][DK] | tk[HB][H] | stat[NWAVE][HB][2] | acc[NWAVE][HB][V]
+  const int KG = TALK ? G : 1;       // key heads a query row meets
+  const int QD = KG * DK;
+  // lds: qs[HB][KG*DK] | stat[NWAVE][HB][2] | acc[NWAVE][HB][V]
   float* qs = lds;
-  float* tk = qs + NQ * DK;
-  float* stat = tk + (TALK ? HB * H : 0);
+  float* stat = qs + HB * QD;
   float* accs = stat + NWAVE * HB * 2;
 
   const int seq = tok_seq[t], pos = tok_pos[t];
   const int* tab = table + (int64_t)seq * P;
-  for (int i = threadIdx.x; i < NQ * DK; i += BLOCK)
-    qs[i] = q[(int64_t)t * H * DK + qbase * DK + i] * scale;
-  if (TALK)
-    for (int i = threadIdx.x; i < HB * H; i += BLOCK)
-      tk[i] = talk[(h0 + i / H) * H + (i % H)];
+  const float* qt = q + (int64_t)t * H * DK;
+  for (int i = threadIdx.x; i < HB * QD; i += BLOCK) {
+    const int b = i / QD, r = i - b * QD;
+    if (!TALK) {
+      qs[i] = qt[(h0 + b) * DK + r] * scale;
+    } else {
+      const int c = r / DK, d = r - c * DK;
+      float acc = 0.f;
+      for (int g = c * rep; g < (c + 1) * rep; ++g)
+        acc += talk[(h0 + b) * H + g] * qt[g * DK + d];
+      qs[i] = acc * scale;
+    }
+  }
   __syncthreads();
 
   float m[HB], l[HB], a[HB][VR];
@@ -144,8 +154,10 @@ __global__ __launch_bounds__(BLOCK) void flex_attn_row_kernel(
 #pragma unroll
     for (int b = 0; b < HB; ++b) s[b] = 0.f;
     if (valid) {
-      if (!TALK) {
-        const TK* kr = kpool + (page_row + (int64_t)g0 * PAGE + lane) * DK;
+      for (int c = 0; c < KG; ++c) {
+        const int g = TALK ? c : g0;
+        const TK* kr = kpool + (page_row + (int64_t)g * PAGE + lane) * DK;
+        const float* qc = qs + c * DK;
         if (vec8) {
           const bf16x8* k8 = reinterpret_cast<const bf16x8*>(kr);
           for (int d8 = 0; d8 < DK / 8; ++d8) {
@@ -155,35 +167,15 @@ __global__ __launch_bounds__(BLOCK) void flex_attn_row_kernel(
               const float kd = bf2f(kk.v[e]);
 #pragma unroll
               for (int b = 0; b < HB; ++b)
-                s[b] += qs[b * DK + d8 * 8 + e] * kd;
+                s[b] += qc[b * QD + d8 * 8 + e] * kd;
             }
           }
         } else {
           for (int d = 0; d < DK; ++d) {
             const float kd = ldv<TK>(kr + d);
 #pragma unroll
-            for (int b = 0; b < HB; ++b) s[b] += qs[b * DK + d] * kd;
+            for (int b = 0; b < HB; ++b) s[b] += qc[b * QD + d] * kd;
           }
-        }
-      } else {
-        for (int hs = 0; hs < H; ++hs) {
-          const TK* kr =
-              kpool + (page_row + (int64_t)(hs / rep) * PAGE + lane) * DK;
-          const float* qh = qs + hs * DK;
-          float raw = 0.f;
-          if (vec8) {
-            const bf16x8* k8 = reinterpret_cast<const bf16x8*>(kr);
-            for (int d8 = 0; d8 < DK / 8; ++d8) {
-              const bf16x8 kk = k8[d8];
-#pragma unroll
-              for (int e = 0; e < 8; ++e)
-                raw += qh[d8 * 8 + e] * bf2f(kk.v[e]);
-            }
-          } else {
-            for (int d = 0; d < DK; ++d) raw += qh[d] * ldv<TK>(kr + d);
-          }
-#pragma unroll
-          for (int b = 0; b < HB; ++b) s[b] += tk[b * H + hs] * raw;
         }
       }
     }
@@ -320,9 +312,8 @@ void launch_rows(bool has_talk, dim3 grid, size_t smem, hipStream_t stream,
                        H, G, DK, V, scale, window, sink);
 }
 
-size_t rows_smem(bool has_talk, int hb, int H, int DK, int V) {
-  return sizeof(float) * ((size_t)(has_talk ? H : hb) * DK +
-                          (has_talk ? (size_t)hb * H : 0) +
+size_t rows_smem(bool has_talk, int hb, int G, int DK, int V) {
+  return sizeof(float) * ((size_t)hb * (has_talk ? G : 1) * DK +
                           (size_t)NWAVE * hb * 2 + (size_t)NWAVE * hb * V);
 }
 
@@ -363,7 +354,7 @@ int tl_flex_attn_heads_per_block(int H, int G, int DK, int V, int has_talk) {
   const int vrr = vr <= 1 ? 1 : vr <= 2 ? 2 : vr <= 4 ? 4 : 8;
   for (int hb = 8; hb >= 1; hb >>= 1) {
     if ((H / G) % hb != 0 || hb * vrr > 32) continue;
-    if (rows_smem(has_talk != 0, hb, H, DK, V) <= 64 * 1024) return hb;
+    if (rows_smem(has_talk != 0, hb, G, DK, V) <= 64 * 1024) return hb;
   }
   return 0;
 }
@@ -380,7 +371,7 @@ int tl_flex_attn_rows(const void* q, const void* kpool, const void* vpool,
   const int hb = tl_flex_attn_heads_per_block(H, G, DK, V, has_talk ? 1 : 0);
   if (hb == 0 || ns < 1 || (ns > 1 && !part)) return 1;
   const int vr = (V + WAVE_SIZE - 1) / WAVE_SIZE;
-  const size_t smem = rows_smem(has_talk, hb, H, DK, V);
+  const size_t smem = rows_smem(has_talk, hb, G, DK, V);
   dim3 grid(T, H / hb, ns);
 #define TL_FA(TT, HBB, VRR)                                                  \
   launch_rows<TT, HBB, VRR>(has_talk, grid, smem, stream, (const float*)q,   \

@@ -18,6 +18,21 @@
 // Tokens are staged in rounds of RT so a round needs three barriers.
 // Shapes whose state does not fit the register budget take the generic
 // kernel, which keeps S in the slot's memory.
+//
+// Long prompt portions take the chunk form instead. With chunks of C
+// tokens, S0 the state before a chunk and i, j indices inside it:
+//     o_i = a^(i+1) S0^T q_i + sum_{j<=i} a^(i-j) (q_i . k_j) v_j
+//     S1  = a^n S0 + sum_j a^(n-1-j) k_j v_j^T           (n tokens in it)
+// so every chunk needs four small matrix products (Q K^T, (A o M) V,
+// Kw^T V, Qd S0), all chunks at once as batched fp32 GEMMs of the vendor
+// library, and only the chain S0 -> S1 over a sequence's chunks is
+// sequential, an elementwise pass. The kernels here do what is not a
+// matrix product: tl_lightning_chunk_prep lays out silu(q), silu(k),
+// silu(v) per (chunk, head), zero-padded, with the decay-weighted copies
+// Qd = a^(i+1) q and Kw = a^(n-1-j) k; tl_lightning_decay_mask applies
+// M[i][j] = a^(i-j) (j <= i, else 0); tl_lightning_chain turns the chunk
+// summaries into the state before each chunk and leaves the final state
+// in the slot. Everything is fp32.
 
 #include "common.hpp"
 
@@ -161,9 +176,133 @@ __global__ __launch_bounds__(BLOCK) void lightning_scan_generic_kernel(
   }
 }
 
+// grid (chunks, H); outputs [chunk][h][C][D|V] fp32, rows >= n are zero
+template <typename T>
+__global__ __launch_bounds__(BLOCK) void lightning_chunk_prep_kernel(
+    const T* __restrict__ proj, int ld, int q_off, int k_off, int v_off,
+    const float* __restrict__ decay, const int* __restrict__ cu_c,
+    float* __restrict__ Qs, float* __restrict__ Qd, float* __restrict__ Ks,
+    float* __restrict__ Kw, float* __restrict__ Vs, int H, int D, int V,
+    int C) {
+  extern __shared__ float pw[];            // a^0 .. a^C
+  const int c = blockIdx.x, h = blockIdx.y;
+  const int t0 = cu_c[c], n = cu_c[c + 1] - t0;
+  const float a = decay[h];
+  for (int i = threadIdx.x; i <= C; i += BLOCK) pw[i] = powf(a, (float)i);
+  __syncthreads();
+  const int64_t base = ((int64_t)c * H + h) * C;
+  for (int i = threadIdx.x; i < C * D; i += BLOCK) {
+    const int r = i / D, d = i - r * D;
+    float qv = 0.f, kv = 0.f, qd = 0.f, kw = 0.f;
+    if (r < n) {
+      const T* row = proj + (int64_t)(t0 + r) * ld;
+      qv = silu(ldf<T>(row + q_off + h * D + d));
+      kv = silu(ldf<T>(row + k_off + h * D + d));
+      qd = qv * pw[r + 1];
+      kw = kv * pw[n - 1 - r];
+    }
+    const int64_t o = (base + r) * D + d;
+    Qs[o] = qv;
+    Qd[o] = qd;
+    Ks[o] = kv;
+    Kw[o] = kw;
+  }
+  for (int i = threadIdx.x; i < C * V; i += BLOCK) {
+    const int r = i / V, e = i - r * V;
+    float vv = 0.f;
+    if (r < n)
+      vv = silu(ldf<T>(proj + (int64_t)(t0 + r) * ld + v_off + h * V + e));
+    Vs[(base + r) * V + e] = vv;
+  }
+}
+
+// A [chunks*H][C][C] in place: A[i][j] *= a^(i-j) for j <= i, else 0
+__global__ __launch_bounds__(BLOCK) void lightning_decay_mask_kernel(
+    float* __restrict__ A, const float* __restrict__ decay, int H, int C) {
+  extern __shared__ float pw[];
+  const int h = blockIdx.x % H;
+  const float a = decay[h];
+  for (int i = threadIdx.x; i < C; i += BLOCK) pw[i] = powf(a, (float)i);
+  __syncthreads();
+  float* Ab = A + (int64_t)blockIdx.x * C * C;
+  for (int i = threadIdx.x; i < C * C; i += BLOCK) {
+    const int r = i / C, j = i - r * C;
+    Ab[i] = j <= r ? Ab[i] * pw[r - j] : 0.f;
+  }
+}
+
+// grid (B, H, ceil(D*V / BLOCK)): U [chunks][H][D*V] holds the chunk
+// summaries on entry and the state BEFORE each chunk on exit; the slot
+// receives the state after the sequence's last chunk.
+__global__ __launch_bounds__(BLOCK) void lightning_chain_kernel(
+    float* __restrict__ U, float* __restrict__ S,
+    const float* __restrict__ decay, const int* __restrict__ cu_c,
+    const int* __restrict__ chunk_base, const int* __restrict__ n_chunks,
+    const int* __restrict__ slots, const int* __restrict__ pos0, int H,
+    int DV) {
+  const int b = blockIdx.x, h = blockIdx.y;
+  const int e = blockIdx.z * BLOCK + threadIdx.x;
+  const int nc = n_chunks[b];
+  if (e >= DV || nc <= 0) return;
+  const float a = decay[h];
+  float* Sp = S + ((int64_t)slots[b] * H + h) * DV + e;
+  float s = pos0[b] == 0 ? 0.f : *Sp;
+  const int c0 = chunk_base[b];
+  for (int c = c0; c < c0 + nc; ++c) {
+    float* up = U + ((int64_t)c * H + h) * DV + e;
+    const float u = *up;
+    *up = s;
+    s = powf(a, (float)(cu_c[c + 1] - cu_c[c])) * s + u;
+  }
+  *Sp = s;
+}
+
 }  // namespace
 
 extern "C" {
+
+void tl_lightning_chunk_prep(const void* proj, int ld, int q_off, int k_off,
+                             int v_off, const void* decay, const void* cu_c,
+                             void* Qs, void* Qd, void* Ks, void* Kw, void* Vs,
+                             int NC, int H, int D, int V, int C, int is_f32,
+                             hipStream_t stream) {
+  if (NC <= 0) return;
+  dim3 grid(NC, H), block(BLOCK);
+  const size_t smem = sizeof(float) * (C + 1);
+  if (is_f32)
+    hipLaunchKernelGGL(lightning_chunk_prep_kernel<float>, grid, block, smem,
+                       stream, (const float*)proj, ld, q_off, k_off, v_off,
+                       (const float*)decay, (const int*)cu_c, (float*)Qs,
+                       (float*)Qd, (float*)Ks, (float*)Kw, (float*)Vs, H, D,
+                       V, C);
+  else
+    hipLaunchKernelGGL(lightning_chunk_prep_kernel<bf16>, grid, block, smem,
+                       stream, (const bf16*)proj, ld, q_off, k_off, v_off,
+                       (const float*)decay, (const int*)cu_c, (float*)Qs,
+                       (float*)Qd, (float*)Ks, (float*)Kw, (float*)Vs, H, D,
+                       V, C);
+}
+
+void tl_lightning_decay_mask(void* A, const void* decay, int NCH, int H,
+                             int C, hipStream_t stream) {
+  if (NCH <= 0) return;
+  hipLaunchKernelGGL(lightning_decay_mask_kernel, dim3(NCH), dim3(BLOCK),
+                     sizeof(float) * C, stream, (float*)A,
+                     (const float*)decay, H, C);
+}
+
+void tl_lightning_chain(void* U, void* S, const void* decay, const void* cu_c,
+                        const void* chunk_base, const void* n_chunks,
+                        const void* slots, const void* pos0, int B, int H,
+                        int DV, hipStream_t stream) {
+  if (B <= 0) return;
+  dim3 grid(B, H, (DV + BLOCK - 1) / BLOCK);
+  hipLaunchKernelGGL(lightning_chain_kernel, grid, dim3(BLOCK), 0, stream,
+                     (float*)U, (float*)S, (const float*)decay,
+                     (const int*)cu_c, (const int*)chunk_base,
+                     (const int*)n_chunks, (const int*)slots,
+                     (const int*)pos0, H, DV);
+}
 
 // returns 0 on success, 1 if the launch cannot be made
 int tl_lightning_scan(const void* proj, int ld, int q_off, int k_off,

@@ -106,6 +106,22 @@ class RaggedMeta:
             self._chunks[size] = hit
         return hit
 
+    def chunk_rows(self, size: int) -> torch.Tensor:
+        """For every flat token its row in the chunk-major layout of
+        ``scan_chunks(size)`` (chunk index * size + offset in the chunk):
+        int64 [T] on the device."""
+        hit = self.__dict__.setdefault("_chunk_rows", {}).get(size)
+        if hit is None:
+            rows, c = [], 0
+            for b in range(self.B):
+                for o in range(0, self.new_h[b], size):
+                    n = min(size, self.new_h[b] - o)
+                    rows += range(c * size, c * size + n)
+                    c += 1
+            hit = torch.tensor(rows, dtype=torch.int64).to(self._device)
+            self._chunk_rows[size] = hit
+        return hit
+
     @property
     def last_rows(self) -> List[int]:
         """Flat index of every sequence's last token."""
@@ -507,8 +523,8 @@ def flex_attention(q: torch.Tensor, kpool: torch.Tensor,
         # the step's shape only
         span = min(meta.max_kv, window) if window > 0 else meta.max_kv
         n_split = 1
-        while (n_split < 16 and meta.T * H * n_split < 1024
-               and span > 512 * n_split):
+        while (n_split < 16 and meta.T * H * n_split < 2048
+               and span > 256 * n_split):
             n_split *= 2
         return _ext().flex_attn_rows(q, kpool, vpool, meta.tok_seq,
                                      meta.tok_pos, meta.table, talk, int(H),
@@ -563,6 +579,30 @@ def lightning_scan(proj: torch.Tensor, offs, decay: torch.Tensor,
     q_off, k_off, v_off = offs
     T = proj.shape[0]
     if proj.is_cuda:
+        chunk = SCAN_CHUNK
+        while meta.T * H * D * V * 4 // chunk > (1 << 31):
+            chunk *= 2                   # bound the chunk-state scratch
+        if (max(meta.new_h) >= 4 * chunk
+                and not os.environ.get("TL_NO_SCAN_CHUNKS")):
+            # long prompt portions: chunk form. Per chunk the intra-chunk
+            # part (Q K^T with the decay mask, times V), the chunk summary
+            # Kw^T V and the carried part Qd S0 are batched fp32 GEMMs over
+            # all chunks at once; only the chain of summaries is sequential.
+            C = _ext()
+            cu_c, _, _, base, cnt, nc, _ = meta.scan_chunks(chunk)
+            Qs, Qd, Ks, Kw, Vs = C.lightning_chunk_prep(
+                proj, int(q_off), int(k_off), int(v_off), decay, cu_c,
+                int(H), int(D), int(V), chunk)
+            A = torch.bmm(Qs, Ks.transpose(1, 2))
+            C.lightning_decay_mask_(A, decay)
+            O = torch.bmm(A, Vs)
+            U = torch.bmm(Kw.transpose(1, 2), Vs)
+            C.lightning_chain_(U, S, decay, cu_c, base, cnt, meta.slots,
+                               meta.pos0)
+            O.baddbmm_(Qd, U)
+            rows = meta.chunk_rows(chunk)
+            return O.view(nc, H, chunk, V).transpose(1, 2).reshape(
+                nc * chunk, H * V).index_select(0, rows)
         return _ext().lightning_scan(proj, int(q_off), int(k_off),
                                      int(v_off), decay, S, meta.cu,
                                      meta.slots, meta.pos0, int(H), int(D),
