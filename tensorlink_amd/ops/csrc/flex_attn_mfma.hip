@@ -135,8 +135,10 @@ __global__ __launch_bounds__(256) void flex_attn_tile_kernel(
   const int vchunks = V / 8;                // 16-byte chunks per value row
   for (int k0 = k_begin; k0 < k_end; k0 += KT) {
     __syncthreads();                        // previous round's reads done
+    // lane -> key fastest: the 2-byte transposed stores of a wave then
+    // fall into consecutive LDS words instead of a few banks
     for (int i = threadIdx.x; i < KT * vchunks; i += 256) {
-      const int kk = i / vchunks, c8 = i - kk * vchunks;
+      const int c8 = i / KT, kk = i - c8 * KT;
       const int j = min(k0 + kk, k_end - 1);
       const int page = tab[j / PAGE];
       const bf16x8 v8 = *reinterpret_cast<const bf16x8*>(
