@@ -72,6 +72,13 @@ __global__ __launch_bounds__(BLOCK) void rms_scale_kernel(
   }
 }
 
+DEVINLINE float gelu_f(float z, int tanh_form) {
+  if (tanh_form)
+    return 0.5f * z *
+           (1.f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+  return 0.5f * z * (1.f + erff(z * 0.7071067811865476f));
+}
+
 template <typename T>
 __global__ __launch_bounds__(BLOCK) void gelu_kernel(
     const T* __restrict__ x, T* __restrict__ out, int64_t n, int N,
@@ -79,19 +86,27 @@ __global__ __launch_bounds__(BLOCK) void gelu_kernel(
     const int* __restrict__ tokens) {
   for (int64_t i = (int64_t)blockIdx.x * BLOCK + threadIdx.x; i < n;
        i += (int64_t)gridDim.x * BLOCK) {
-    const float z = ldf<T>(x, i);
-    float v;
-    if (tanh_form)
-      v = 0.5f * z *
-          (1.f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
-    else
-      v = 0.5f * z * (1.f + erff(z * 0.7071067811865476f));
+    float v = gelu_f(ldf<T>(x, i), tanh_form);
     if (table) {
       const int64_t r = i / N;
       const int c = (int)(i - r * N);
       v *= ldf<T>(table, (int64_t)tokens[r] * ldt + table_col + c);
     }
     stf<T>(out, i, v);
+  }
+}
+
+// bf16, no gathered factor, n a multiple of 8: 16-byte loads and stores
+__global__ __launch_bounds__(BLOCK) void gelu_vec8_kernel(
+    const bf16x8* __restrict__ x, bf16x8* __restrict__ out, int64_t n8,
+    int tanh_form) {
+  for (int64_t i = (int64_t)blockIdx.x * BLOCK + threadIdx.x; i < n8;
+       i += (int64_t)gridDim.x * BLOCK) {
+    const bf16x8 a = x[i];
+    bf16x8 r;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) r.v[e] = f2bf(gelu_f(bf2f(a.v[e]), tanh_form));
+    out[i] = r;
   }
 }
 
@@ -145,6 +160,12 @@ void tl_gelu(const void* x, void* out, int64_t n, int N, int tanh_form,
              const void* table, int ldt, int table_col, const void* tokens,
              int is_f32, hipStream_t stream) {
   if (n <= 0) return;
+  if (!is_f32 && !table && n % 8 == 0) {
+    hipLaunchKernelGGL(gelu_vec8_kernel, dim3(ew_grid(n / 8)), dim3(BLOCK), 0,
+                       stream, (const bf16x8*)x, (bf16x8*)out, n / 8,
+                       tanh_form);
+    return;
+  }
   dim3 grid(ew_grid(n)), block(BLOCK);
   if (is_f32)
     hipLaunchKernelGGL(gelu_kernel<float>, grid, block, 0, stream,

@@ -581,6 +581,11 @@ def test_rowwise_ops(device, dtype):
     tok = torch.randint(0, 20, (T,), generator=g, dtype=torch.int32)
     assert torch.allclose(mx.gelu(z.to(device)).float().cpu().double(),
                           O.gelu_erf(z.double()), atol=a, rtol=a)
+    z8 = torch.randn(16, 24, generator=g).to(dtype) * 2   # 16-byte path
+    for tanh_form, fn in ((False, O.gelu_erf), (True, O.gelu_tanh)):
+        got = mx.gelu(z8.to(device), tanh_form)
+        assert torch.allclose(got.float().cpu().double(), fn(z8.double()),
+                              atol=a, rtol=a)
     got = mx.gelu(z.to(device), True, table=table.to(device),
                   tokens=tok.to(device), table_col=5)
     want = O.gelu_tanh(z.double()) * table[tok.long(), 5:15].double()
