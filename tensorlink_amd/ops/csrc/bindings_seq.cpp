@@ -32,7 +32,7 @@ int tl_flex_attn_rows(const void* q, const void* kpool, const void* vpool,
                       const void* table, int P, const void* talk, void* out,
                       int out_f32, void* part, int ns, int T, int H, int G,
                       int DK, int V, float scale, int window, int sink,
-                      int pool_f32, hipStream_t stream);
+                      int pool_f32, int hb_max, hipStream_t stream);
 int tl_flex_attn_tiles_ok(int H, int G, int KG, int DK, int V);
 void tl_stage_queries(const void* q, const void* talk, void* out, int T,
                       int H, int G, int DK, hipStream_t stream);
@@ -221,7 +221,7 @@ Tensor flex_attn_rows(Tensor q, Tensor kpool, c10::optional<Tensor> vpool,
                       Tensor tok_seq, Tensor tok_pos, Tensor table,
                       c10::optional<Tensor> talk, int64_t H, double scale,
                       int64_t window, bool sink, int64_t V, bool out_f32,
-                      int64_t n_split) {
+                      int64_t n_split, int64_t hb_max) {
   SEQ_F32(q);
   SEQ_IN(kpool);
   SEQ_I32(tok_seq);
@@ -273,7 +273,7 @@ Tensor flex_attn_rows(Tensor q, Tensor kpool, c10::optional<Tensor> vpool,
       talk.has_value() ? talk->data_ptr() : nullptr, out.data_ptr(),
       out_f32 ? 1 : 0, n_split > 1 ? part.data_ptr() : nullptr, (int)n_split,
       (int)T, (int)H, G, DK, (int)V, (float)scale, (int)window, sink ? 1 : 0,
-      pool_f32, seq_stream());
+      pool_f32, (int)std::max<int64_t>(1, hb_max), seq_stream());
   TORCH_CHECK(rc == 0, "flex_attn_rows: launch refused");
   return out;
 }

@@ -194,18 +194,28 @@ __global__ __launch_bounds__(BLOCK) void flex_attn_row_kernel(
     }
     const int jb = max(0, lo - j0), je = min(WAVE_SIZE, pos + 1 - j0);
     const TK* vtile = vpool + (page_row + (int64_t)g0 * PAGE) * vld;
-    for (int jj = jb; jj < je; ++jj) {
-      float w[HB];
+    // eight keys' value rows are loaded before they are used, so their
+    // latencies overlap instead of adding up
+    for (int jj0 = jb; jj0 < je; jj0 += 8) {
+      float vv[8][VR];
 #pragma unroll
-      for (int b = 0; b < HB; ++b) w[b] = __shfl(p[b], jj, WAVE_SIZE);
-      const TK* vr = vtile + (int64_t)jj * vld;
+      for (int u = 0; u < 8; ++u) {
+        const TK* vr = vtile + (int64_t)(jj0 + u) * vld;
 #pragma unroll
-      for (int r = 0; r < VR; ++r) {
-        const int c = lane + r * WAVE_SIZE;
-        if (c < V) {
-          const float vv = ldv<TK>(vr + c);
+        for (int r = 0; r < VR; ++r) {
+          const int c = lane + r * WAVE_SIZE;
+          vv[u][r] = (jj0 + u < je && c < V) ? ldv<TK>(vr + c) : 0.f;
+        }
+      }
 #pragma unroll
-          for (int b = 0; b < HB; ++b) a[b][r] += w[b] * vv;
+      for (int u = 0; u < 8; ++u) {
+        // lanes past the range hold weight 0
+        const int jj = min(jj0 + u, WAVE_SIZE - 1);
+#pragma unroll
+        for (int b = 0; b < HB; ++b) {
+          const float w = jj0 + u < je ? __shfl(p[b], jj, WAVE_SIZE) : 0.f;
+#pragma unroll
+          for (int r = 0; r < VR; ++r) a[b][r] += w * vv[u][r];
         }
       }
     }
@@ -348,27 +358,35 @@ void tl_norm_rope_rows(const void* src, int ld, int col, int n_heads,
 
 // heads per block for a shape: the largest of 8, 4, 2, 1 that divides the
 // heads per key group and fits the register and LDS budgets; 0 if none
-int tl_flex_attn_heads_per_block(int H, int G, int DK, int V, int has_talk) {
+static int heads_per_block(int H, int G, int DK, int V, int has_talk,
+                           int hb_max) {
   if (V > 512 || G <= 0 || H % G != 0) return 0;
   const int vr = (V + WAVE_SIZE - 1) / WAVE_SIZE;
   const int vrr = vr <= 1 ? 1 : vr <= 2 ? 2 : vr <= 4 ? 4 : 8;
   for (int hb = 8; hb >= 1; hb >>= 1) {
+    if (hb > hb_max && hb > 1) continue;
     if ((H / G) % hb != 0 || hb * vrr > 32) continue;
     if (rows_smem(has_talk != 0, hb, G, DK, V) <= 64 * 1024) return hb;
   }
   return 0;
 }
 
-// returns 0 on success, 1 if the shape is outside what the kernel serves
+int tl_flex_attn_heads_per_block(int H, int G, int DK, int V, int has_talk) {
+  return heads_per_block(H, G, DK, V, has_talk, 8);
+}
+
+// returns 0 on success, 1 if the shape is outside what the kernel serves.
+// hb_max caps the heads per block: few rows (decoding) want many small
+// blocks, many rows want the key and value loads shared by more heads.
 int tl_flex_attn_rows(const void* q, const void* kpool, const void* vpool,
                       int vld, const void* tok_seq, const void* tok_pos,
                       const void* table, int P, const void* talk, void* out,
                       int out_f32, void* part, int ns, int T, int H, int G,
                       int DK, int V, float scale, int window, int sink,
-                      int pool_f32, hipStream_t stream) {
+                      int pool_f32, int hb_max, hipStream_t stream) {
   if (T <= 0) return 0;
   const bool has_talk = talk != nullptr;
-  const int hb = tl_flex_attn_heads_per_block(H, G, DK, V, has_talk ? 1 : 0);
+  const int hb = heads_per_block(H, G, DK, V, has_talk ? 1 : 0, hb_max);
   if (hb == 0 || ns < 1 || (ns > 1 && !part)) return 1;
   const int vr = (V + WAVE_SIZE - 1) / WAVE_SIZE;
   const size_t smem = rows_smem(has_talk, hb, G, DK, V);

@@ -530,7 +530,7 @@ def flex_attention(q: torch.Tensor, kpool: torch.Tensor,
                                      meta.tok_pos, meta.table, talk, int(H),
                                      float(scale), int(window), bool(sink),
                                      int(V), out_dtype == torch.float32,
-                                     n_split)
+                                     n_split, 1 if meta.T * H <= 512 else 8)
     out = torch.empty(T, H, V)
     qf = q.view(T, H, DK)
     rep = H // G
