@@ -708,6 +708,78 @@ def test_greedy_generation(tmp_path_factory, device, dtype):
     assert out[0].tolist()[:keep] == want[0][:keep]
 
 
+def random_cfg(rng):
+    """A random model of the design: 2-5 layers in any order, 1-9 heads,
+    head sizes from 8 to 136 (below, at and above a wave's 64 columns, not
+    all multiples of 8), windows from 1 to beyond the sequence, shared
+    latents, optional feed-forward, token input and soft cap."""
+    w = rng.choice([24, 40, 64, 96])
+    layers, lat_src = [], None
+    for i in range(rng.randint(2, 5)):
+        kind = rng.choice(["lightning", "latent_attention", "attention"])
+        if kind == "lightning":
+            H = rng.randint(1, 5)
+            mc = lit(H, rng.choice([8, 16, 24, 40, 72]),
+                     rng.choice([8, 24, 48, 64, 136]),
+                     [rng.choice([1.0, 0.999, 0.97, 0.9, 0.5])
+                      for _ in range(H)])
+        elif kind == "latent_attention":
+            if lat_src is not None and rng.random() < 0.5:
+                src = layers[lat_src]["mixer"]
+                mc = lat(rng.randint(1, 6), rng.choice([8, 16, 40]),
+                         src["rot_dim"], rng.choice([8, 16, 40]),
+                         src["kv_rank"], base=src["rot"]["base"],
+                         kv_from=lat_src)
+            else:
+                mc = lat(rng.randint(1, 6), rng.choice([8, 16, 40]),
+                         rng.choice([2, 4, 8, 16]), rng.choice([8, 16, 40]),
+                         rng.choice([8, 16, 48, 72, 130]),
+                         base=rng.choice([100.0, 10000.0]))
+                lat_src = i
+        else:
+            G, rep = rng.randint(1, 3), rng.choice([1, 2, 3, 4])
+            D = rng.choice([8, 16, 24, 48, 96])
+            mc = att(G * rep, G, D, rng.choice([8, 16, 48, 96, 130]),
+                     min(D, rng.choice([0, 2, 4, 8, D])),
+                     rng.choice([1, 5, 33, 64, 100, 128, 129, 1000]),
+                     base=rng.choice([500.0, 50000.0]))
+        mlp = ({"kind": "dense", "ff": rng.choice([16, 72, 128])}
+               if rng.random() < 0.7 else None)
+        layers.append({"type": kind, "mixer": mc, "mlp": mlp})
+    cfg = {"architecture": "Senulix", "vocab": rng.choice([37, 64, 200]),
+           "width": w, "norm": {"eps": rng.choice([1e-5, 1e-6])},
+           "layers": layers}
+    if rng.random() < 0.7:
+        cfg["token_side"] = {"dim": rng.choice([1, 4, 8, 16])}
+    if rng.random() < 0.7:
+        cfg["logit_softcap"] = rng.choice([5.0, 15.0, 50.0])
+    return cfg
+
+
+@pytest.mark.parametrize("device,dtype", [CPU32, GPU32])
+def test_random_configurations(tmp_path, device, dtype):
+    """Other sizes, orders and constants: whole, portioned and decoded
+    against the oracle. The typical position is held tightly; the worst
+    loosely, since a window whose weight nearly all falls to the sink
+    leaves a tiny output whose direction the output norm amplifies."""
+    import random
+    for seed in (1, 3, 5, 6):
+        cfg = random_cfg(random.Random(seed))
+        P = make_weights(cfg, seed)
+        d = str(tmp_path / f"r{seed}")
+        write_checkpoint(d, cfg, P)
+        toks = tokens(cfg, 140, seed)
+        want = O.forward(cfg, P, toks)
+        runner = PipelineRunner(plan_for_world(d, 1), 0, 1,
+                                device=torch.device(device),
+                                init="checkpoint", ckpt_dir=d, dtype=dtype)
+        for cuts in ([140], [90, 2, 3, 40]):
+            got = run_schedule(batcher(runner, max_ctx=256), toks, cuts)
+            e = rel_err(got, want)
+            assert float(e.median()) < 2e-5 and float(e.max()) < 1e-3, \
+                (seed, cuts, float(e.median()), float(e.max()))
+
+
 # --------------------------------------------------- configuration, loader
 def test_registry_and_strict_loading(tmp_path):
     from tensorlink_amd.models.configs import ModelConfig
